@@ -11,6 +11,9 @@
 * ``query``      stage 2 only for one metapath string (``test_generate_query.py``)
 * ``state``      stage 3 only for one entity (``test_check_state.py``)
 * ``token-probe`` token accounting over two runs (``test_token.py``)
+* ``trace-run``  replay a recorded schedule of token ids through the engine and
+                 write the logits of the wanted positions (engine/trace.py; also
+                 ``bin/trace_run``)
 * ``serve``      OpenAI-Assistants-shaped REST API over the engine, plus the
                  Neo4j HTTP ``/db/{metagraph,stategraph}/tx/commit`` endpoint over
                  the graphs (api/http.py);
@@ -265,6 +268,11 @@ def cmd_serve(args) -> int:
     return 0
 
 
+def cmd_trace_run(args) -> int:
+    from .engine import trace
+    return trace.main(args.model, args.dtype, args.out, args.max_tokens, args.device)
+
+
 def main(argv: Optional[List[str]] = None) -> int:
     p = argparse.ArgumentParser(prog="k8s_llm_rca_amd", description=__doc__,
                                 formatter_class=argparse.RawDescriptionHelpFormatter)
@@ -324,6 +332,14 @@ def main(argv: Optional[List[str]] = None) -> int:
     sp.add_argument("--host", default="127.0.0.1")
     sp.add_argument("--port", type=int, default=8000)
     sp.set_defaults(fn=cmd_serve)
+    sp = sub.add_parser("trace-run", help="replay a schedule of token ids (JSON lines on stdin), write logits")
+    sp.add_argument("--model", required=True, help="checkpoint folder (config.json + model.safetensors)")
+    sp.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    sp.add_argument("--out", required=True, help="folder for <step>.f32")
+    sp.add_argument("--max-tokens", type=int, required=True, help="tokens the page pool holds")
+    sp.add_argument("--device", default=None, help="default: cuda when there is one")
+    sp.add_argument("-v", "--verbose", action="store_true")
+    sp.set_defaults(fn=cmd_trace_run)
     args = p.parse_args(argv)
     logging.basicConfig(level=logging.INFO if args.verbose else logging.WARNING)
     return args.fn(args)

@@ -53,12 +53,9 @@ from .types import PART_MIN, SPEC, EngineConfig, InFlight, Request, Sequence  # 
 log = logging.getLogger(__name__)
 
 
-def _build_model(mc: ModelConfig, device, dtype, pc, seed):
-    if mc.arch == "opt":
-        from ..models.opt import OPTModel
-        return OPTModel(mc, device, dtype, seed=seed)
-    from ..models.llama import LlamaModel
-    return LlamaModel(mc, device, dtype, pc, seed=seed)
+def _build_model(mc, device, dtype, pc, seed):
+    from ..models.registry import build_model
+    return build_model(mc, device, dtype, pc, seed)
 
 
 class LLMEngine(SchedulerMixin, StepExecMixin, GraphRunnerMixin, SamplerMixin):
@@ -75,13 +72,14 @@ class LLMEngine(SchedulerMixin, StepExecMixin, GraphRunnerMixin, SamplerMixin):
         self.device = torch.device(cfg.device)
         t0 = time.perf_counter()
         if cfg.weights and model is None:
-            from ..models.llama import LlamaModel
-            from ..models.weights import config_from_hf, load_safetensors
-            self.mc = config_from_hf(cfg.weights)
-            model = LlamaModel(self.mc, self.device, cfg.dtype, self.pc, init=False)
-            load_safetensors(model, cfg.weights)
+            from ..models.registry import load_model
+            model = load_model(cfg.weights, self.device, cfg.dtype, self.pc)  # the class config.json names
+            self.mc = model.cfg
+        elif model is not None and getattr(getattr(model, "cfg", None), "arch", None) == "zasapel":
+            self.mc = model.cfg  # built by the caller from its own configuration
         else:
-            self.mc = get_config(cfg.model, **cfg.model_overrides)
+            from ..models.registry import get_any_config
+            self.mc = get_any_config(cfg.model, **(cfg.model_overrides or {}))
         self.max_context = cfg.max_context or self.mc.max_position
         self.model = model or _build_model(self.mc, self.device, cfg.dtype, self.pc, cfg.seed)
         if hasattr(self.model, "logits_f32"):
@@ -111,10 +109,14 @@ class LLMEngine(SchedulerMixin, StepExecMixin, GraphRunnerMixin, SamplerMixin):
         self.grt = GrammarRuntime(self.tok, self.mc.vocab_size)
         self.eos_ids = [self.tok.eot_id, self.tok.eos_id]
         BS = cfg.block_size
-        nkv, D = self.model.nkv, self.model.D
+        # a model with a cache layout of its own (latent pages, state slots) declares it
+        own_cache = hasattr(self.model, "make_cache")
+        self.stateful = bool(getattr(self.model, "stateful", False))
+        nkv, D = (1, 0) if own_cache else (self.model.nkv, self.model.D)
         nb = cfg.num_blocks
         if nb is None:
-            per = KVPool.bytes_per_block(self.mc.n_layers, nkv, D, BS)
+            per = (self.model.cache_bytes_per_block(BS) if own_cache
+                   else KVPool.bytes_per_block(self.mc.n_layers, nkv, D, BS))
             if self.device.type == "cuda":
                 free, _ = torch.cuda.mem_get_info(self.device)
                 budget = free * cfg.kv_mem_fraction - self._workspace_bytes()
@@ -123,13 +125,20 @@ class LLMEngine(SchedulerMixin, StepExecMixin, GraphRunnerMixin, SamplerMixin):
             if cfg.kv_max_gb is not None:
                 budget = min(budget, cfg.kv_max_gb * (1 << 30))
             nb = max(16, int(budget // per))
-        self.kv = KVPool(self.mc.n_layers, nkv, D, nb, BS, self.device, cfg.dtype)
+        self.kv = (self.model.make_cache(nb, BS) if own_cache
+                   else KVPool(self.mc.n_layers, nkv, D, nb, BS, self.device, cfg.dtype))
+        self.states = None
+        if self.stateful:
+            from .kv_cache import StatePool
+            self.states = StatePool(cfg.state_slots, self.model.state_spec(), self.device)
         # KV host tier: idle threads are swapped to page-locked host memory instead
         # of dropped (engine/kv_offload.py).  One engine per device: at TP > 1 the
         # ranks' pools would have to swap in lockstep, which the channel does not carry
         self.kv_host = None
         if cfg.kv_host_gb and cfg.kv_host_gb > 0:
-            if self.pc.tp_size > 1:
+            if own_cache:
+                log.warning("kv_host_gb ignored: the host tier copies K/V pages, not %s's cache", self.mc.name)
+            elif self.pc.tp_size > 1:
                 log.warning("kv_host_gb ignored at TP = %d (host tier is per-device, TP = 1 only)", self.pc.tp_size)
             else:
                 from .kv_offload import KVHostTier
@@ -173,6 +182,10 @@ class LLMEngine(SchedulerMixin, StepExecMixin, GraphRunnerMixin, SamplerMixin):
                              and self.model.vocab_local % 8 == 0)
         # TP: every rank needs the sampled tokens on its device to overlap steps
         self._async = cfg.async_steps and (self.pc.tp_size == 1 or self._dist_sample or self._sim)
+        if self.stateful:
+            # an overlapped step feeds a token that the host may still reject (the request ended):
+            # pages can be rewound by one position, recurrent state cannot
+            self._async = False
         # TP: the vocab-parallel sampler (its own object, tp_sampler.py)
         self.tps = None
         if self._dist_sample:
@@ -213,7 +226,8 @@ class LLMEngine(SchedulerMixin, StepExecMixin, GraphRunnerMixin, SamplerMixin):
                       "recompute_tokens": 0, "kv_read_blocks_sampled": 0, "kv_unique_blocks_sampled": 0,
                       "tiny_chunk_tokens": 0, "swap_outs": 0, "swap_ins": 0}
         # where every thread's KV lives and what happens when HBM runs short (kv_manager.py)
-        self.kvm = KVCacheManager(self.kv, self.kv_host, self.kv_watermark, self._snapshot, self.stats)
+        self.kvm = KVCacheManager(self.kv, self.kv_host, self.kv_watermark, self._snapshot, self.stats,
+                                  states=self.states)
         self._cancels: List[int] = []
         self.error: Optional[BaseException] = None
         self._fault: Optional[str] = None  # a dead communicator: every later request fails at admission
@@ -259,6 +273,9 @@ class LLMEngine(SchedulerMixin, StepExecMixin, GraphRunnerMixin, SamplerMixin):
 
     def _workspace_bytes(self) -> int:
         mc = self.mc
+        if hasattr(self.model, "workspace_bytes"):
+            return int(self.model.workspace_bytes(self.cfg.max_batch_tokens)
+                       + self.cfg.max_decode_seqs * mc.vocab_size * 4)
         t = self.cfg.max_batch_tokens
         act = t * (mc.hidden * 8 + (mc.q_size + 2 * mc.kv_size) * 2 + mc.intermediate * 6)
         if mc.n_experts:

@@ -41,15 +41,23 @@ class KVPool:
         self.L, self.nkv, self.D = n_layers, n_kv, head_dim
         self.num_blocks = num_blocks
         self.block_size = block_size
-        # zero-filled: stale pages never hold NaN (masked keys multiply V by 0)
-        self.k = torch.zeros(n_layers, num_blocks, n_kv, block_size, head_dim, dtype=dtype, device=device)
-        self.v = torch.zeros(n_layers, num_blocks, n_kv, head_dim, block_size, dtype=dtype, device=device)
+        self._alloc_storage(device, dtype)
         self._free: List[int] = list(range(num_blocks - 1, -1, -1))
         self._ref = np.zeros(num_blocks, dtype=np.int32)
         self._key_of: Dict[int, int] = {}   # registered block -> chain key
         self._by_key: Dict[int, int] = {}   # chain key -> block
         self.peak_used = 0
         self._lock = threading.Lock()
+
+    def _alloc_storage(self, device, dtype) -> None:
+        # zero-filled: stale pages never hold NaN (masked keys multiply V by 0)
+        L, nb, nkv, BS, D = self.L, self.num_blocks, self.nkv, self.block_size, self.D
+        self.k = torch.zeros(L, nb, nkv, BS, D, dtype=dtype, device=device)
+        self.v = torch.zeros(L, nb, nkv, D, BS, dtype=dtype, device=device)
+
+    def tensors(self) -> tuple:
+        """What a model's ``forward`` receives after the step inputs."""
+        return (self.k, self.v)
 
     @staticmethod
     def bytes_per_block(n_layers: int, n_kv: int, head_dim: int, block_size: int, elem: int = 2) -> int:
@@ -126,3 +134,50 @@ class KVPool:
 
     def utilization(self) -> float:
         return 1.0 - len(self._free) / max(1, self.num_blocks)
+
+
+class LatentKVPool(KVPool):
+    """The same page allocator over LATENT pages: one tensor ``c[i]`` of shape
+    ``[num_blocks, block_size, ranks[i]]`` per layer that projects its own
+    key-value latent (layers that attend over another layer's latents hold none).
+    A page index means the same token range in every tensor."""
+
+    def __init__(self, ranks: List[int], num_blocks: int, block_size: int, device, dtype=torch.bfloat16):
+        self.ranks = list(ranks)
+        super().__init__(len(ranks), 1, max(ranks) if ranks else 0, num_blocks, block_size, device, dtype)
+
+    def _alloc_storage(self, device, dtype) -> None:
+        self.k = self.v = None
+        self.c = [torch.zeros(self.num_blocks, self.block_size, r, dtype=dtype, device=device) for r in self.ranks]
+
+    def tensors(self) -> tuple:
+        return (self.c,)
+
+
+class StatePool:
+    """Fixed-size per-sequence state beside the pages: ``slots`` slots of every
+    tensor a model declares (``spec``: name -> shape behind the slot dimension),
+    fp32.  A sequence holds one slot while it has cached tokens; a slot is not
+    cleared when it is handed out again -- kernels read state only past a
+    sequence's first position."""
+
+    def __init__(self, slots: int, spec: Dict[str, Tuple[int, ...]], device):
+        self.slots = slots
+        self.t: Dict[str, torch.Tensor] = {k: torch.zeros((slots,) + tuple(shape), dtype=torch.float32, device=device)
+                                           for k, shape in spec.items()}
+        self._free: List[int] = list(range(slots - 1, -1, -1))
+
+    @property
+    def free_slots(self) -> int:
+        return len(self._free)
+
+    def alloc(self) -> Optional[int]:
+        return self._free.pop() if self._free else None
+
+    def release(self, slot: int) -> None:
+        if slot in self._free or not 0 <= slot < self.slots:
+            raise RuntimeError(f"state slot {slot} released twice or never taken")
+        self._free.append(slot)
+
+    def bytes(self) -> int:
+        return sum(t.numel() * 4 for t in self.t.values())

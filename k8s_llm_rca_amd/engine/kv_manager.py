@@ -31,13 +31,41 @@ from .types import Sequence
 
 class KVCacheManager:
     def __init__(self, pool: KVPool, host=None, watermark: int = 0,
-                 snapshot: Callable[[], List[Sequence]] = list, stats: Optional[Dict] = None):
+                 snapshot: Callable[[], List[Sequence]] = list, stats: Optional[Dict] = None, states=None):
         self.pool = pool
         self.host = host                # KVHostTier or None
         self.watermark = watermark      # swap ahead while free + in-flight pages are below this
         self.snapshot = snapshot        # the engine's sequences (thread-safe copy)
         self.stats = stats if stats is not None else Counter()  # standalone: counters start at 0
         self.BS = pool.block_size
+        # stateful models: the slots of per-sequence recurrent state (kv_cache.StatePool).
+        # State cannot be rewound or shared: a sequence that loses its pages loses its
+        # slot, and a prompt that diverges from the cached tokens restarts from token 0
+        self.states = states
+
+    # ------------------------------------------------------------ state slots
+    def _free_slot(self, s: Sequence) -> None:
+        if self.states is not None and s.slot is not None:
+            self.states.release(s.slot)
+            s.slot = None
+
+    def _ensure_slot(self, s: Sequence, protect: set) -> bool:
+        """A state slot for ``s``, taken from the least recently used idle sequence if none is free."""
+        if self.states is None or s.slot is not None:
+            return True
+        if not self.states.free_slots:
+            for v in sorted((v for v in self.snapshot() if v.req is None and v.slot is not None
+                             and v.id not in protect), key=lambda v: v.last_used):
+                self.drop(v)
+                self.stats["evictions"] += 1
+                break
+        s.slot = self.states.alloc()
+        if s.slot is None:
+            return False
+        if s.n_cached:  # cached tokens without their state cannot be continued
+            self.pool.release(s.blocks)
+            s.blocks, s.bh, s.n_cached = [], [], 0
+        return True
 
     # ------------------------------------------------------------ admission
     def keep_prefix(self, s: Sequence, lcp: int) -> None:
@@ -45,6 +73,8 @@ class KVCacheManager:
         first ``lcp`` (``s.n_cached`` is already ``lcp``): keep those pages and
         give up the rest.  A swapped thread starts its swap-in here."""
         BS = self.BS
+        if self.states is not None and lcp == 0:
+            self._free_slot(s)  # nothing cached any more: the slot goes back until the sequence runs
         del s.bh[lcp // BS:]
         keep = (lcp + BS - 1) // BS
         if s.host is not None:  # swapped to the host tier: bring the kept pages back
@@ -66,6 +96,8 @@ class KVCacheManager:
     def ensure_blocks(self, s: Sequence, upto: int, protect: set) -> bool:
         """Pages for ``s``'s first ``upto`` tokens, making room if needed
         (never at the expense of a sequence in ``protect``)."""
+        if not self._ensure_slot(s, protect):
+            return False
         need = (upto + self.BS - 1) // self.BS - len(s.blocks)
         if need <= 0:
             return True
@@ -92,6 +124,7 @@ class KVCacheManager:
             s.blocks = []
             s.bh = []
             s.n_cached = 0
+            self._free_slot(s)
             self.stats["evictions"] += 1
             if freed >= n_blocks:
                 return
@@ -112,6 +145,7 @@ class KVCacheManager:
             v.blocks = []
             v.bh = []
             v.n_cached = 0
+            self._free_slot(v)
             self.stats["preemptions"] += 1
             if self.ensure_blocks(s, upto, protect):
                 return True
@@ -131,6 +165,7 @@ class KVCacheManager:
             s.host = None
         s.bh = []
         s.n_cached = 0
+        self._free_slot(s)
 
     # ------------------------------------------------------------ prefix sharing
     def attach_prefix(self, s: Sequence) -> None:

@@ -92,6 +92,8 @@ class SchedulerMixin:
             cur = s.tokens
             while lcp < n and cur[lcp] == toks[lcp]:
                 lcp += 1
+            if self.stateful and lcp < s.n_cached:
+                lcp = 0  # recurrent state cannot be rewound to the common prefix: start over
             # cached positions the new prompt re-prefills (history truncation, divergence)
             self.stats["recompute_tokens"] += max(0, n - lcp)
             s.tokens = toks
@@ -218,7 +220,8 @@ class SchedulerMixin:
             if len(s.tokens) > self.kv.num_blocks * BS:
                 self._fail_req(s.req, "context longer than the whole KV pool")
                 continue
-            if self.cfg.prefix_sharing and s.n_cached % BS == 0 and len(s.blocks) == s.n_cached // BS:
+            if (self.cfg.prefix_sharing and not self.stateful and s.n_cached % BS == 0
+                    and len(s.blocks) == s.n_cached // BS):
                 self.kvm.attach_prefix(s)
                 q = min(s.pending, budget)
             if not (self.kvm.ensure_blocks(s, s.n_cached + q, protect)
@@ -276,7 +279,7 @@ class SchedulerMixin:
                 spec_pos[s.id] = s.n_cached
             s.n_cached += q
             s.last_used = time.perf_counter()
-        if self.cfg.prefix_sharing:
+        if self.cfg.prefix_sharing and not self.stateful:
             for s, _ in chunks:  # publish the pages this prefill completed (their KV write is enqueued)
                 self.kvm.register_blocks(s)
         self.stats["steps"] += 1
@@ -312,3 +315,51 @@ class SchedulerMixin:
             else:
                 self._process_tokens(self._launch_sample(*pend))
         return True
+
+    # ------------------------------------------------------- teacher-forced steps
+    def feed(self, entries: List[Tuple[int, List[int], List[int]]]) -> torch.Tensor:
+        """One step with GIVEN next tokens instead of sampled ones: ``entries`` =
+        (sequence id, its next tokens, offsets among them whose logits are wanted).
+        All entries run as one batch through the same packing, cache manager and
+        forward as :meth:`step` -- single tokens and short portions as
+        decode-attention rows, longer portions as prefill chunks -- and the
+        sequences advance by their tokens.  Returns fp32 logits [wanted, vocab]
+        in the order of ``entries``.  For replaying a recorded schedule; no
+        request is attached and nothing is sampled."""
+        if self._pending_sample is not None:
+            raise RuntimeError("feed() while a sampled step is in flight")
+        if self._releases:
+            self._apply_releases()
+        with self._lock:
+            seqs = [self.seqs[sid] for sid, _, _ in entries]
+        protect = set(s.id for s in seqs)
+        BS = self.kv.block_size
+        tiny, big, decode = [], [], []
+        for s, (_, toks, _) in zip(seqs, entries):
+            if not toks:
+                raise ValueError("an entry without tokens")
+            if s.n_cached != len(s.tokens):
+                raise RuntimeError(f"sequence {s.id} has tokens that were never run")
+            s.tokens.extend(int(t) for t in toks)
+            q = len(toks)
+            if len(s.tokens) > self.kv.num_blocks * BS or not self.kvm.ensure_blocks(s, s.n_cached + q, protect):
+                raise MemoryError("KV pool exhausted")
+            (decode if q == 1 else tiny if q <= self.cfg.tiny_chunk_tokens else big).append((s, q))
+        if len(decode) + sum(q for _, q in tiny) > max(self.cfg.max_decode_seqs, 1):
+            tiny, big = [], tiny + big
+        drows = [(s, 0) for s, _ in decode] + [(s, j) for s, q in tiny for j in range(q)]
+        rows = decode + tiny + big
+        row0, off = {}, 0
+        for s, q in rows:
+            row0[s.id] = off
+            off += q
+        want_rows = [row0[s.id] + int(w) for s, (_, _, want) in zip(seqs, entries) for w in want]
+        logits = self._forward(drows, big, want_rows)
+        now = time.perf_counter()
+        for s, q in rows:
+            s.n_cached += q
+            s.last_used = now
+        self.stats["steps"] += 1
+        self.stats["prefill_tokens"] += sum(q for _, q in tiny + big)
+        self.stats["decode_tokens"] += len(decode)
+        return logits.float()

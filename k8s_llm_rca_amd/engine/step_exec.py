@@ -120,6 +120,7 @@ class StepExecMixin:
         if spec is not None and self._chan is not None:
             _spec_tok(spec)  # TP: sample(k) -- a message + an all-gather -- goes before forward(k+1) on every rank
         if (not chunks and self.cfg.use_graphs and self.device.type == "cuda" and decode and self._graphs_ok()
+                and getattr(self.model, "graph_capturable", True)
                 and self.kv.block_size % 64 == 0):
             out = self._forward_graph(decode, spec, sample_idx)
             self.stats["graph_steps"] += 1
@@ -194,8 +195,82 @@ class StepExecMixin:
     # = ids[T] pos[T] slots[T] sidx[ns] | bt_d ctx_d qs_d | bt_p ctx_p qs_p tseq ttok0 tlen
     HDR = 14
 
+    def _pack_segments(self, decode, chunks, sample_idx):
+        """The step in the SEGMENT layout (models with ``step_layout == "segments"``):
+        consecutive rows of one sequence form a segment -- a decode token, the tokens
+        of a short portion among the decode rows, or a prefill chunk -- with its first
+        position, its state slot and its block table; attention, convolutions and
+        recurrences all address rows through it.  Header tag 2; payload
+        ids pos slots sidx | row_seg seg_row0 seg_pos0 seg_slot block_tables."""
+        BS = self.kv.block_size
+        segs: List[Tuple[Sequence, int, int]] = []   # (sequence, offset past n_cached, rows)
+        for s, j in decode:
+            if segs and segs[-1][0] is s and segs[-1][1] + segs[-1][2] == j:
+                segs[-1] = (s, segs[-1][1], segs[-1][2] + 1)
+            else:
+                segs.append((s, j, 1))
+        n_dec_rows = len(decode)
+        segs += [(s, 0, q) for s, q in chunks]
+        n = len(segs)
+        maxb = max(len(s.blocks) for s, _, _ in segs)
+        bt = np.zeros((n, maxb), dtype=np.int32)
+        row0 = np.zeros(n + 1, dtype=np.int32)
+        pos0 = np.zeros(n, dtype=np.int32)
+        slot = np.zeros(n, dtype=np.int32)
+        ids, pos, slots, row_seg = [], [], [], []
+        for i, (s, j, q) in enumerate(segs):
+            a = s.n_cached + j
+            bt[i, :len(s.blocks)] = s.blocks
+            row0[i + 1] = row0[i] + q
+            pos0[i] = a
+            if s.slot is None:
+                raise RuntimeError(f"sequence {s.id} runs without a state slot")
+            slot[i] = s.slot
+            ids.extend(s.tokens[a:a + q])
+            p = np.arange(a, a + q, dtype=np.int64)
+            pos.append(p)
+            slots.append(np.asarray(s.blocks, dtype=np.int64)[p // BS] * BS + p % BS)
+            row_seg.append(np.full(q, i, dtype=np.int32))
+        T = int(row0[-1])
+        arrays = [np.asarray(ids, dtype=np.int32), np.concatenate(pos).astype(np.int32),
+                  np.concatenate(slots).astype(np.int32), np.asarray(sample_idx, dtype=np.int32),
+                  np.concatenate(row_seg), row0, pos0, slot, bt]
+        flat = np.concatenate([x.reshape(-1).astype(np.int32, copy=False) for x in arrays])
+        header = np.zeros(self.HDR, dtype=np.int64)
+        header[:7] = [2, flat.size, T, n_dec_rows, n, maxb, len(sample_idx)]
+        return header, flat
+
+    def _exec_segments(self, header: np.ndarray, flat_host: np.ndarray, flat_dev: torch.Tensor):
+        from ..models.zasapel import SegStepInputs
+        from ..ops.seq_ops import SegMeta
+        _, _, T, n_dec_rows, n, maxb, ns = [int(v) for v in header[:7]]
+        o = 0
+
+        def take(k):
+            nonlocal o
+            d, h = flat_dev[o:o + k], flat_host[o:o + k]
+            o += k
+            return d, h
+
+        d_ids, _ = take(T)
+        d_pos, _ = take(T)
+        d_slots, _ = take(T)
+        d_sidx, _ = take(ns)
+        row_seg, _ = take(T)
+        row0, row0_h = take(n + 1)
+        pos0, pos0_h = take(n)
+        slot, slot_h = take(n)
+        bt, _ = take(n * maxb)
+        seg = SegMeta(n_seg=n, row_seg=row_seg, seg_row0=row0, seg_pos0=pos0, seg_slot=slot,
+                      block_tables=bt.view(n, maxb), row0_host=row0_h.tolist(), pos0_host=pos0_h.tolist(),
+                      slot_host=slot_h.tolist(), n_single=n_dec_rows)
+        inp = SegStepInputs(d_ids, d_pos, d_slots, seg, d_sidx.long())
+        return self.model.forward(inp, *self.kv.tensors(), self.states.t)
+
     def _pack_step(self, decode, chunks, sample_idx):
         """``decode``: decode-attention rows (sequence, token offset past n_cached)."""
+        if getattr(self.model, "step_layout", None) == "segments":
+            return self._pack_segments(decode, chunks, sample_idx)
         ids_d, pos_d, slots_d = self._decode_token_arrays(decode)
         ids, pos, slots = self._token_arrays(list(chunks))
         ids, pos, slots = np.concatenate([ids_d, ids]), np.concatenate([pos_d, pos]), np.concatenate([slots_d, slots])
@@ -234,6 +309,10 @@ class StepExecMixin:
         """Build StepInputs from the wire format and run the forward (every TP rank)."""
         from ..models.llama import StepInputs
 
+        if int(header[0]) == 2:
+            if spec is not None:
+                raise RuntimeError("segment-layout steps take their tokens from the host")
+            return self._exec_segments(header, flat_host, flat_dev)
         (_, _, T, nd, n_dec, maxb_d, n_pre, maxb_p, n_tiles, ns, n_parts, n_merge, part,
          n_items) = [int(v) for v in header]
         if self._sim:

@@ -122,6 +122,9 @@ class EngineConfig:
     # below this many (None: one max-size prefill step plus one full thread)
     kv_host_watermark: Optional[int] = None
     model_overrides: dict = field(default_factory=dict)
+    # stateful models: how many sequences can hold recurrent state at once
+    # (a sequence without cached tokens needs none)
+    state_slots: int = 64
 
 
 class Request:
@@ -148,7 +151,7 @@ class Request:
 
 
 class Sequence:
-    __slots__ = ("id", "tokens", "n_cached", "blocks", "req", "last_used", "bh", "host", "loading")
+    __slots__ = ("id", "tokens", "n_cached", "blocks", "req", "last_used", "bh", "host", "loading", "slot")
 
     def __init__(self, sid: int):
         self.id = sid
@@ -164,6 +167,9 @@ class Sequence:
         # swap-in still on the copy stream (the sequence is not scheduled before)
         self.host: Optional[List[int]] = None
         self.loading = None
+        # stateful models (recurrent layers, short convolutions): the state slot that
+        # holds what the first n_cached tokens left behind (kv_cache.StatePool)
+        self.slot: Optional[int] = None
 
     @property
     def pending(self) -> int:

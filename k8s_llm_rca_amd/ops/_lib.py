@@ -82,6 +82,18 @@ _SIGS = {
     "k8s_set_knob": [I, I],
     "k8s_nonfinite_flag": [P, ctypes.c_long, P, P],
     "k8s_get_knob": [I],
+    "k8s_embed_sinpos": [P, P, P, P, I, I, F, I, P],
+    "k8s_canon_conv": [P, P, P, P, P, P, P, P, I, I, I, I, I, P],
+    "k8s_mingru_scan": [P, P, P, P, P, P, P, P, I, I, I, P],
+    "k8s_postnorm": [P, P, I, P, I, P, I, I, F, F, P],
+    "k8s_latent_norm": [P, I, P, P, P, P, P, I, I, I, F, I, P],
+    "k8s_latent_attn_rows": [P, P, P, I, P, P, P, P, I, P, I, I, I, I, I, F, I, P],
+    "k8s_polynorm": [P, P, P, I, I, F, I, P],
+    "k8s_glu_clamp": [P, P, I, I, F, F, F, I, P],
+    "k8s_router": [P, P, I, I, I, I, I, I, P, P, I, P],
+    "k8s_moe_gather": [P, P, P, P, I, I, I, I, P],
+    "k8s_moe_combine_f32": [P, P, P, P, I, I, I, I, P],
+    "k8s_grouped_any": [P, P, P, P, I, I, I, I, I, P],
     "k8s_walks": [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P, P, P, P],
 }
 # entry points whose C return type is not int

@@ -71,7 +71,7 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, fuse_s
         out = torch.empty(rows, N, dtype=a.dtype, device=a.device)
     if rows == 0:
         return out
-    if glds and use_hip(a) and not fuse_silu and N % 64 == 0 and K % (64 * splits) == 0:
+    if glds and use_hip(a) and a.dtype == torch.bfloat16 and not fuse_silu and N % 64 == 0 and K % (64 * splits) == 0:
         # the LDS-DMA strip kernel (csrc/kernels/gemm_stream.hip grouped_glds_kernel)
         assert a.dtype == torch.bfloat16 and w.is_contiguous() and a.stride(1) == 1 and out.is_contiguous()
         max_tiles = (rows + 63) // 64 + E
@@ -79,7 +79,7 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, fuse_s
         check(lib().k8s_grouped_glds(ptr(a), a.stride(0), ptr(w), ptr(out), out.stride(0), ptr(offsets), E, N, K,
                                      max_tiles, glds, splits, ptr(part), rows, stream_ptr(a)), "grouped_glds")
         return out
-    if use_hip(a) and N % 128 == 0 and K % (64 * splits) == 0:
+    if use_hip(a) and a.dtype == torch.bfloat16 and N % 128 == 0 and K % (64 * splits) == 0:
         assert a.dtype == torch.bfloat16 and w.is_contiguous() and a.stride(1) == 1 and out.is_contiguous()
         assert a.shape[1] == (2 * K if fuse_silu else K)
         max_tiles = (rows + 63) // 64 + E
@@ -87,6 +87,12 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, fuse_s
         check(lib().k8s_grouped_gemm(ptr(a), a.stride(0), ptr(w), ptr(out), out.stride(0), ptr(offsets), E, N, K,
                                      max_tiles, int(fuse_silu), splits, ptr(part), rows, stream_ptr(a)),
               "grouped_gemm")
+        return out
+    if use_hip(a) and not fuse_silu and a.dtype == w.dtype and a.dtype in (torch.bfloat16, torch.float32):
+        # any shape, bf16 or fp32, offsets read on the device (csrc/kernels/ffn_ops.hip)
+        assert w.is_contiguous() and a.is_contiguous() and out.is_contiguous() and a.shape[1] == K
+        check(lib().k8s_grouped_any(ptr(a), ptr(w), ptr(offsets), ptr(out), rows, E, N, K,
+                                    0 if a.dtype == torch.bfloat16 else 1, stream_ptr(a)), "grouped_any")
         return out
     offs = offsets.tolist()
     for e in range(E):
@@ -144,3 +150,80 @@ def _split_scratch(dev: torch.device, n: int) -> torch.Tensor:
 def reserve_split_scratch(dev: torch.device, max_rows: int, N: int, splits: int) -> None:
     """Allocate the split-K partial buffer before any HIP-graph capture."""
     _split_scratch(dev, max_rows * N * splits)
+
+
+# ------------------------------------------------------------------ routers and gated units beside Mixtral's
+def _dt(t: torch.dtype) -> int:
+    return 0 if t == torch.bfloat16 else 1
+
+
+def route_direct(h: torch.Tensor, w_router: torch.Tensor, k: int, scoring: str = "sigmoid",
+                 renorm: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Router straight from the hidden rows: fp32 logits ``h @ w_router.T``, scores by ``scoring``
+    ("sigmoid" or "softmax"), the ``k`` largest (ties: lowest index), renormalised to sum 1 only
+    with ``renorm``.  Returns (weights fp32 [T, k], ids int32 [T, k])."""
+    T, W = h.shape
+    E = w_router.shape[0]
+    if use_hip(h):
+        assert h.is_contiguous() and w_router.is_contiguous() and h.dtype == w_router.dtype
+        w = torch.empty(T, k, dtype=torch.float32, device=h.device)
+        ids = torch.empty(T, k, dtype=torch.int32, device=h.device)
+        check(lib().k8s_router(ptr(h), ptr(w_router), T, W, E, k, 0 if scoring == "sigmoid" else 1, int(renorm),
+                               ptr(w), ptr(ids), _dt(h.dtype), stream_ptr(h)), "router")
+        return w, ids
+    z = h.float() @ w_router.float().t()
+    s = torch.sigmoid(z) if scoring == "sigmoid" else torch.softmax(z, -1)
+    # stable descending sort: equal scores keep the lower expert first
+    order = torch.sort(s, dim=-1, descending=True, stable=True).indices[:, :k]
+    w = torch.gather(s, 1, order)
+    if renorm:
+        w = w / w.sum(-1, keepdim=True)
+    return w, order.int()
+
+
+def gather_rows(h: torch.Tensor, order: torch.Tensor, k: int, w: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Rows of ``h`` in expert order (``order`` from :func:`align`), each scaled by its routing weight
+    ``w`` [T, k] when the weight multiplies the expert's input."""
+    n, W = order.numel(), h.shape[1]
+    if use_hip(h):
+        assert h.is_contiguous() and (w is None or (w.dtype == torch.float32 and w.is_contiguous()))
+        xp = torch.empty(n, W, dtype=h.dtype, device=h.device)
+        check(lib().k8s_moe_gather(ptr(h), ptr(order), ptr(w), ptr(xp), n, W, k, _dt(h.dtype), stream_ptr(h)),
+              "moe_gather")
+        return xp
+    xp = h.float()[(order // k).long()]
+    if w is not None:
+        xp = xp * w.reshape(-1)[order.long()][:, None]
+    return xp.to(h.dtype)
+
+
+def glu_clamp(gu: torch.Tensor, alpha: float, limit: float, up_shift: float = 1.0) -> torch.Tensor:
+    """Clamped gated unit on ``gu`` [rows, 2F] = (gate | up): ``g = min(gate, limit)``,
+    ``u = clamp(up, -limit, limit)``, result ``g * sigmoid(alpha g) * (u + up_shift)``."""
+    rows, F2 = gu.shape
+    F = F2 // 2
+    if use_hip(gu):
+        assert gu.is_contiguous()
+        out = torch.empty(rows, F, dtype=gu.dtype, device=gu.device)
+        check(lib().k8s_glu_clamp(ptr(gu), ptr(out), rows, F, float(alpha), float(limit), float(up_shift),
+                                  _dt(gu.dtype), stream_ptr(gu)), "glu_clamp")
+        return out
+    g = gu[:, :F].float().clamp(max=limit)
+    u = gu[:, F:].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + up_shift)).to(gu.dtype)
+
+
+def combine_f32(y_perm: torch.Tensor, inv: torch.Tensor, T: int, k: int,
+                w: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 ``out[t] = sum_j (w[t, j] or 1) * y_perm[inv[t k + j]]``."""
+    W = y_perm.shape[1]
+    if use_hip(y_perm):
+        assert y_perm.is_contiguous()
+        out = torch.empty(T, W, dtype=torch.float32, device=y_perm.device)
+        check(lib().k8s_moe_combine_f32(ptr(y_perm), ptr(inv), ptr(w), ptr(out), T, W, k, _dt(y_perm.dtype),
+                                        stream_ptr(y_perm)), "moe_combine_f32")
+        return out
+    g = y_perm.float()[inv.long()].view(T, k, W)
+    if w is not None:
+        g = g * w.view(T, k, 1)
+    return g.sum(1)

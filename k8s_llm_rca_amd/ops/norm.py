@@ -76,3 +76,22 @@ def nonfinite_flag(x: torch.Tensor, flag: torch.Tensor) -> None:
         return
     if not torch.isfinite(x).all():
         flag[0] = 1
+
+
+def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
+    """PolyNorm activation of fp32 rows: ``a N(z) + b N(z^2) + c N(z^3) + e`` with ``coef = (a, b, c, e)``,
+    powers element by element and ``N(v) = v / sqrt(mean(v^2) + eps)`` over the row."""
+    T, F = z.shape
+    out = torch.empty(T, F, dtype=out_dtype, device=z.device)
+    if use_hip(z):
+        assert z.dtype == torch.float32 and z.is_contiguous() and coef.dtype == out_dtype and coef.numel() == 4
+        check(lib().k8s_polynorm(ptr(z), ptr(coef), ptr(out), T, F, float(eps), 0 if out_dtype == torch.bfloat16 else 1,
+                                 stream_ptr(z)), "polynorm")
+        return out
+    a, b, c, e = [float(v) for v in coef.float()]
+
+    def unit(v):
+        return v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+
+    out.copy_((a * unit(z) + b * unit(z * z) + c * unit(z * z * z) + e).to(out_dtype))
+    return out

@@ -1,0 +1,195 @@
+"""Ops of layers that carry per-sequence state besides the paged cache:
+sinusoidal positions, the short causal convolution in front of a sublayer, the
+minGRU recurrence, the post-sublayer norm of an fp32 residual, and attention
+over a paged latent cache (``csrc/kernels/seq_ops.hip``, ``latent_attn.hip``).
+
+A step's rows come in SEGMENTS (:class:`SegMeta`): consecutive rows of one
+sequence -- a decode token or a portion of a prompt.  Device tensors run the HIP
+kernels; CPU tensors the fp32 PyTorch forms below (the engine's CPU backend).
+The residual stream, norms, recurrence and softmax are fp32 in both; ``dt`` is
+the activation / weight type (bf16 or fp32).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional
+
+import torch
+
+from ._lib import check, lib, ptr, stream_ptr, use_hip
+
+
+@dataclass
+class SegMeta:
+    n_seg: int
+    row_seg: torch.Tensor      # [T] int32: segment of every row
+    seg_row0: torch.Tensor     # [n_seg + 1] int32 row offsets
+    seg_pos0: torch.Tensor     # [n_seg] int32 position of the segment's first token
+    seg_slot: torch.Tensor     # [n_seg] int32 state slot of the segment's sequence
+    block_tables: torch.Tensor  # [n_seg, maxb] int32 cache pages
+    row0_host: List[int]
+    pos0_host: List[int]
+    slot_host: List[int]
+    # rows [0, n_single) are one-token segments (decode kernels); the rest portions of prompts
+    n_single: int = 0
+
+
+def _dt(t: torch.dtype) -> int:
+    if t == torch.bfloat16:
+        return 0
+    if t == torch.float32:
+        return 1
+    raise TypeError(f"activations must be bfloat16 or float32, not {t}")
+
+
+def embed_sinpos(ids: torch.Tensor, pos: torch.Tensor, embed: torch.Tensor, base: float = 10000.0) -> torch.Tensor:
+    """fp32 ``embed[ids] + sinusoid(pos)``: entry 2i = sin(p base^(-2i/W)), entry 2i+1 its cosine."""
+    T, W = ids.shape[0], embed.shape[1]
+    if use_hip(embed):
+        x = torch.empty(T, W, dtype=torch.float32, device=embed.device)
+        check(lib().k8s_embed_sinpos(ptr(ids), ptr(pos), ptr(embed), ptr(x), T, W, float(base), _dt(embed.dtype),
+                                     stream_ptr(embed)), "embed_sinpos")
+        return x
+    i2 = (torch.arange(W, dtype=torch.float64) // 2) * 2
+    ang = pos.double()[:, None] * torch.exp(-i2 / W * torch.log(torch.tensor(float(base), dtype=torch.float64)))[None]
+    pe = torch.where((torch.arange(W) % 2 == 1)[None], ang.cos(), ang.sin()).float()
+    return embed[ids.long()].float() + pe
+
+
+def canon_conv(x: torch.Tensor, w: torch.Tensor, tail: torch.Tensor, seg: SegMeta, out_dtype) -> torch.Tensor:
+    """``h = x + conv(x)``: per channel ``conv(x)_t = sum_j w[:, j] x_(t - taps + 1 + j)`` over each sequence
+    (zeros before its start).  ``tail`` [slots, taps - 1, W] fp32 holds every sequence's last inputs and is
+    advanced by this step's rows."""
+    T, W = x.shape
+    taps = w.shape[1]
+    h = torch.empty(T, W, dtype=out_dtype, device=x.device)
+    if use_hip(x):
+        assert x.dtype == torch.float32 and x.is_contiguous() and w.is_contiguous() and tail.is_contiguous()
+        assert tail.shape[1:] == (taps - 1, W) and w.dtype == out_dtype and taps <= 16
+        check(lib().k8s_canon_conv(ptr(x), ptr(w), ptr(tail), ptr(seg.row_seg), ptr(seg.seg_row0), ptr(seg.seg_pos0),
+                                   ptr(seg.seg_slot), ptr(h), T, seg.n_seg, W, taps, _dt(out_dtype), stream_ptr(x)),
+              "canon_conv")
+        return h
+    wf = w.float()
+    nt = taps - 1
+    for s in range(seg.n_seg):
+        a, b, p0, sl = seg.row0_host[s], seg.row0_host[s + 1], seg.pos0_host[s], seg.slot_host[s]
+        prev = tail[sl] if p0 > 0 else torch.zeros(nt, W)
+        ext = torch.cat([prev, x[a:b]])                     # inputs pos0 - nt .. pos0 + n - 1
+        acc = x[a:b].clone()
+        for j in range(taps):
+            acc += wf[:, j] * ext[j:j + (b - a)]
+        h[a:b] = acc.to(out_dtype)
+        if nt:
+            tail[sl] = ext[-nt:]
+    return h
+
+
+def mingru_scan(zug: torch.Tensor, bz: torch.Tensor, bu: torch.Tensor, state: torch.Tensor, seg: SegMeta,
+                out_dtype) -> torch.Tensor:
+    """minGRU over every segment: ``zug`` [T, 3C] fp32 = (z | u | g) projections without biases;
+    ``S <- (1 - z) S + z cand`` with ``z = sigmoid(.)``, ``cand = u + 1/2`` for ``u >= 0`` else ``sigmoid(u)``;
+    returns ``S * silu(g)``.  ``state`` [slots, C] fp32 is read (past position 0) and advanced."""
+    T, C3 = zug.shape
+    C = C3 // 3
+    y = torch.empty(T, C, dtype=out_dtype, device=zug.device)
+    if use_hip(zug):
+        assert zug.dtype == torch.float32 and zug.is_contiguous() and state.is_contiguous() and bz.dtype == out_dtype
+        check(lib().k8s_mingru_scan(ptr(zug), ptr(bz), ptr(bu), ptr(state), ptr(seg.seg_row0), ptr(seg.seg_pos0),
+                                    ptr(seg.seg_slot), ptr(y), seg.n_seg, C, _dt(out_dtype), stream_ptr(zug)),
+              "mingru_scan")
+        return y
+    z = torch.sigmoid(zug[:, :C] + bz.float())
+    u = zug[:, C:2 * C] + bu.float()
+    g = zug[:, 2 * C:]
+    cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+    for s in range(seg.n_seg):
+        a, b, p0, sl = seg.row0_host[s], seg.row0_host[s + 1], seg.pos0_host[s], seg.slot_host[s]
+        S = state[sl].clone() if p0 > 0 else torch.zeros(C)
+        for r in range(a, b):
+            S = (1 - z[r]) * S + z[r] * cand[r]
+            y[r] = (S * torch.nn.functional.silu(g[r])).to(out_dtype)
+        state[sl] = S
+    return y
+
+
+def postnorm_(x: torch.Tensor, y: torch.Tensor, w: torch.Tensor, alpha: float, eps: float) -> torch.Tensor:
+    """In place on the fp32 residual: ``x <- unit_rms(alpha x + y) * (1 + w)``."""
+    T, W = x.shape
+    if use_hip(x):
+        assert x.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous() and y.shape == x.shape
+        check(lib().k8s_postnorm(ptr(x), ptr(y), _dt(y.dtype), ptr(w), _dt(w.dtype), None, T, W, float(alpha),
+                                 float(eps), stream_ptr(x)), "postnorm")
+        return x
+    v = alpha * x + y.float()
+    x.copy_(v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * (1.0 + w.float()))
+    return x
+
+
+def unit_norm_out(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
+    """``unit_rms(x) * (1 + w)`` of fp32 rows as activations of ``w``'s type (``x`` is left as it is)."""
+    T, W = x.shape
+    out = torch.empty(T, W, dtype=w.dtype, device=x.device)
+    if use_hip(x):
+        assert x.dtype == torch.float32 and x.is_contiguous()
+        check(lib().k8s_postnorm(ptr(x), None, 1, ptr(w), _dt(w.dtype), ptr(out), T, W, 1.0, float(eps),
+                                 stream_ptr(x)), "unit_norm_out")
+        return out
+    out.copy_((x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * (1.0 + w.float())).to(w.dtype))
+    return out
+
+
+def latent_norm(dn: torch.Tensor, wq: torch.Tensor, wkv: Optional[torch.Tensor], slots: torch.Tensor,
+                cache: Optional[torch.Tensor], q_rank: int, kv_rank: int, eps: float, out_dtype) -> torch.Tensor:
+    """Rows of the joint down projection ``dn`` [T, >= q_rank + kv_rank] fp32: the query latent is
+    RMS-normed (plain weight) and returned; the key-value latent (``wkv`` given) is RMS-normed and
+    written to the paged latent ``cache`` [pages, BS, kv_rank] at ``slots`` (page * BS + offset)."""
+    T = dn.shape[0]
+    cq = torch.empty(T, q_rank, dtype=out_dtype, device=dn.device)
+    kr = kv_rank if wkv is not None else 0
+    if use_hip(dn):
+        assert dn.dtype == torch.float32 and dn.stride(1) == 1 and wq.dtype == out_dtype
+        assert cache is None or (cache.is_contiguous() and cache.dtype == out_dtype and cache.shape[-1] == kv_rank)
+        check(lib().k8s_latent_norm(ptr(dn), dn.stride(0), ptr(wq), ptr(wkv), ptr(slots), ptr(cq), ptr(cache), T,
+                                    q_rank, kr, float(eps), _dt(out_dtype), stream_ptr(dn)), "latent_norm")
+        return cq
+    q = dn[:, :q_rank]
+    cq.copy_((q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * wq.float()).to(out_dtype))
+    if kr:
+        c = dn[:, q_rank:q_rank + kr]
+        c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * wkv.float()
+        ok = slots >= 0
+        cache.view(-1, kr)[slots[ok].long()] = c[ok].to(cache.dtype)
+    return cq
+
+
+def latent_attention(qa: torch.Tensor, cache: torch.Tensor, gate: torch.Tensor, seg: SegMeta, scale: float,
+                     out_dtype) -> torch.Tensor:
+    """Causal attention of absorbed queries ``qa`` [T, H, R] fp32 over the paged latents ``cache``
+    [pages, BS, R]: ``p = softmax(scale * qa . c_j)`` over the keys up to the row's own position,
+    output ``sigmoid(gate[t, h]) * sum_j p_j c_j`` [T, H, R] (``gate`` fp32, row stride free)."""
+    T, H, R = qa.shape
+    BS = cache.shape[1]
+    out = torch.empty(T, H, R, dtype=out_dtype, device=qa.device)
+    if use_hip(qa):
+        assert qa.dtype == torch.float32 and qa.is_contiguous() and cache.is_contiguous() and cache.dtype == out_dtype
+        assert gate.dtype == torch.float32 and gate.stride(1) == 1 and gate.shape[1] >= H
+        assert seg.block_tables.is_contiguous()
+        check(lib().k8s_latent_attn_rows(ptr(qa), ptr(cache), ptr(seg.block_tables), seg.block_tables.shape[1],
+                                         ptr(seg.row_seg), ptr(seg.seg_row0), ptr(seg.seg_pos0), ptr(gate),
+                                         gate.stride(0), ptr(out), 0, T, H, R, BS, float(scale), _dt(out_dtype),
+                                         stream_ptr(qa)), "latent_attn_rows")
+        return out
+    flat = cache.view(-1, R)
+    for s in range(seg.n_seg):
+        a, b, p0 = seg.row0_host[s], seg.row0_host[s + 1], seg.pos0_host[s]
+        n_ctx = p0 + b - a
+        pages = seg.block_tables[s].long()
+        kp = torch.arange(n_ctx)
+        c = flat[pages[kp // BS] * BS + kp % BS].float()                      # [ctx, R]
+        sc = torch.einsum("thr,jr->thj", qa[a:b], c) * scale
+        vis = kp[None, :] <= (p0 + torch.arange(b - a))[:, None]
+        sc = sc.masked_fill(~vis[:, None, :], float("-inf"))
+        o = torch.einsum("thj,jr->thr", torch.softmax(sc, -1), c)
+        out[a:b] = (o * torch.sigmoid(gate[a:b, :H])[:, :, None]).to(out_dtype)
+    return out
