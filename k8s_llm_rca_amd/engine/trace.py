@@ -28,7 +28,9 @@ def make_engine(model_dir: str, dtype: torch.dtype, max_tokens: int, device: Opt
     """An engine over the checkpoint in ``model_dir`` whose page pool holds ``max_tokens`` tokens
     (each live request rounded up to whole pages) and ``state_slots`` sequences' state."""
     if device is None:
-        device = "cuda" if torch.cuda.is_available() else "cpu"
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU: the replay runs the HIP kernels (pass --device cpu for the reference ops)")
+        device = "cuda"
     if device.startswith("cuda"):
         torch.backends.cuda.matmul.allow_tf32 = False   # float32 means float32
         torch.backends.cudnn.allow_tf32 = False

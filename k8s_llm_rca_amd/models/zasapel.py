@@ -360,8 +360,7 @@ class ZasapelModel:
                 S.postnorm_(x, y, L["norm2"], cfg.postln_alpha, cfg.rms_eps)
             if layers_out is not None:
                 layers_out.append(x.clone())
-        T = x.shape[0]
-        sel = x.index_select(0, inp.logits_idx) if inp.logits_idx.numel() != T else x
+        sel = x.index_select(0, inp.logits_idx)   # wanted rows in the caller's order (any permutation)
         yn = S.unit_norm_out(sel.contiguous(), self.final_norm, cfg.rms_eps)
         return self._lin32(yn, self.lm_head)
 
