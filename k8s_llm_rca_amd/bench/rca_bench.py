@@ -719,6 +719,10 @@ def spawn_ranks(n: int, argv: List[str]) -> int:
 
 def main(argv=None) -> int:
     argv = list(sys.argv[1:] if argv is None else argv)
+    if any(a.startswith("--model-throughput") for a in argv):
+        # prefill / decode tokens/s of model presets side by side (bench/model_bench.py)
+        from . import model_bench
+        return model_bench.main(argv)
     p = parser()
     pre, _ = p.parse_known_args(argv)
     if pre.preset:

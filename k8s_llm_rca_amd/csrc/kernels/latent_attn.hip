@@ -152,3 +152,256 @@ K8S_API int k8s_latent_attn_rows(const float* qa, const void* cache, const int* 
   }
   return (int)hipGetLastError();
 }
+
+namespace k8s {
+
+// ---------------------------------------------------------------------------
+// MFMA form (bf16): v_mfma_f32_16x16x32_bf16, one wave per work item, no LDS.
+//
+// The latents are cached twice: c [pages][BS][R] (a key's R numbers contiguous:
+// the QK^T operand) and ct [pages][R][BS] (8 consecutive keys of one latent
+// column contiguous: the PV operand), as the K / transposed-V pages of the
+// head-wise attention kernels.  A wave owns MT tiles of 16 query rows; a tile is
+// TPM consecutive tokens x HC heads (HC = min(H, 16), TPM = 16 / HC), so all its
+// rows read the same keys.  Keys go in chunks of 32 (never across a page:
+// BS % 32 == 0).  Swapped QK^T (S^T = C Q^T): a lane owns ONE query row
+// (lane & 15) and 8 of its key scores; MFMA row rho of key tile t holds key
+// 8 (rho >> 2) + 4 t + (rho & 3), so lane quarter h ends with keys 8h .. 8h + 7,
+// the k-slots of the PV operand: P moves from accumulator to operand in place.
+//
+// Items ([n][4] int32: segment, first row, tokens, position of the first row's
+// token) are made on the host from the step's segments.  SPLIT (decode rows):
+// grid.y partitions of `part` keys write unnormalised partials which
+// latent_reduce merges -- the partition borders depend on the key index only,
+// never on the batch.  Otherwise (prompt portions) a wave walks every key its
+// rows see and writes the gated, normalised output.
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct LatArgs {
+  const uint16_t* qa;     // [T][H][R] bf16
+  const uint16_t* c;      // [pages][BS][R]
+  const uint16_t* ct;     // [pages][R][BS]
+  const int* bt;
+  int maxb;
+  const int* items;
+  int n_items;
+  const float* gate;
+  int ldg;
+  uint16_t* out;          // [T][H][R]
+  float* part_o;          // [T][H][n_parts][R]
+  float* part_ml;         // [T][H][n_parts][2]
+  int n_parts, part;
+  int H, HC, TPM, BS;
+  float scale_log2;
+};
+
+__device__ __forceinline__ bf16x8 ld16(const uint16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+
+template <int NR, int MT, bool SPLIT>
+__global__ void __launch_bounds__(256) latent_attn_mfma_kernel(LatArgs a) {
+  constexpr int R = NR * 32, ND = R / 16;
+  const int lane = threadIdx.x & 63, r = lane & 15, h = lane >> 4;
+  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= a.n_items) return;
+  const int sg = a.items[item * 4], row0 = a.items[item * 4 + 1], ntok = a.items[item * 4 + 2],
+            pos0 = a.items[item * 4 + 3];
+  const int hc = blockIdx.z;
+  int k_begin = 0, k_end = pos0 + ntok;
+  if constexpr (SPLIT) {
+    k_begin = blockIdx.y * a.part;
+    k_end = min(k_end, k_begin + a.part);
+    if (k_begin >= k_end) return;
+  }
+  // this lane's query row in every tile
+  const int tl = r / a.HC, hl = r - tl * a.HC, head = hc * a.HC + hl;
+  bf16x8 qf[MT][NR];
+  int limit[MT];
+  f32x4 o[MT][ND];
+  float m[MT], l[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int ti = mt * a.TPM + tl;
+    const bool valid = tl < a.TPM && ti < ntok && head < a.H;
+    limit[mt] = valid ? min(pos0 + ti + 1, k_end) : 0;
+    const uint16_t* qp = a.qa + ((size_t)(row0 + (valid ? ti : 0)) * a.H + (valid ? head : 0)) * R;
+#pragma unroll
+    for (int cc = 0; cc < NR; ++cc) {
+      qf[mt][cc] = ld16(qp + 32 * cc + 8 * h);
+      if (!valid)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) qf[mt][cc][j] = (__bf16)0.f;
+    }
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt) o[mt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m[mt] = -INFINITY;
+    l[mt] = 0.f;
+  }
+  const int* pages = a.bt + (size_t)sg * a.maxb;
+  for (int kb = k_begin & ~31; kb < k_end; kb += 32) {
+    const int page = pages[kb / a.BS], off = kb % a.BS;
+    const uint16_t* cp = a.c + (size_t)page * a.BS * R;
+    const uint16_t* tp = a.ct + (size_t)page * R * a.BS;
+    bf16x8 kf[2][NR];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int key = off + 8 * (r >> 2) + 4 * t + (r & 3);
+#pragma unroll
+      for (int cc = 0; cc < NR; ++cc) kf[t][cc] = ld16(cp + (size_t)key * R + 32 * cc + 8 * h);
+    }
+    bf16x8 pf[MT];
+    float ar[MT][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      float p[8];
+      float cmax = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int cc = 0; cc < NR; ++cc) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][cc], qf[mt][cc], s, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = kb + 8 * h + 4 * t + i;
+          const float v = (key < limit[mt] && key >= k_begin) ? s[i] * a.scale_log2 : -INFINITY;
+          p[4 * t + i] = v;
+          cmax = fmaxf(cmax, v);
+        }
+      }
+      cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
+      cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
+      const float mnew = fmaxf(m[mt], cmax);
+      const float alpha = (mnew == -INFINITY) ? 1.f : exp2f(m[mt] - mnew);
+      float psum = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float e = (mnew == -INFINITY) ? 0.f : exp2f(p[j] - mnew);
+        psum += e;
+        pf[mt][j] = (__bf16)e;
+      }
+      l[mt] = l[mt] * alpha + psum;
+      m[mt] = mnew;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ar[mt][i] = __shfl(alpha, 4 * h + i, 64);
+    }
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt) {
+      const bf16x8 vf = ld16(tp + (size_t)(16 * dt + r) * a.BS + off + 8 * h);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[mt][dt][i] *= ar[mt][i];
+        o[mt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf[mt], vf, o[mt][dt], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    float lt = l[mt];
+    lt += __shfl_xor(lt, 16, 64);
+    lt += __shfl_xor(lt, 32, 64);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int q = 4 * h + i;                       // the query row of accumulator element i
+      const int qtl = q / a.HC, qhl = q - qtl * a.HC, qhead = hc * a.HC + qhl, ti = mt * a.TPM + qtl;
+      const float lq = __shfl(lt, q, 64), mq = __shfl(m[mt], q, 64);
+      if (!(qtl < a.TPM && ti < ntok && qhead < a.H)) continue;
+      const size_t rh = (size_t)(row0 + ti) * a.H + qhead;
+      if constexpr (SPLIT) {
+        const size_t pi = rh * a.n_parts + blockIdx.y;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) a.part_o[pi * R + 16 * dt + r] = o[mt][dt][i];
+        if (r == 0) {
+          a.part_ml[pi * 2] = mq;
+          a.part_ml[pi * 2 + 1] = lq;
+        }
+      } else {
+        const float g = 1.f / (1.f + expf(-a.gate[(size_t)(row0 + ti) * a.ldg + qhead]));
+        const float sc = lq > 0.f ? g / lq : 0.f;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) a.out[rh * R + 16 * dt + r] = f2bf(o[mt][dt][i] * sc);
+      }
+    }
+  }
+}
+
+// Merge of the key partitions of decode rows: one workgroup per (row, head).
+// A row at position p has ceil((p + 1) / part) partitions.
+__global__ void __launch_bounds__(128) latent_reduce_kernel(const float* __restrict__ part_o,
+                                                            const float* __restrict__ part_ml,
+                                                            const int* __restrict__ positions,
+                                                            const float* __restrict__ gate, int ldg,
+                                                            uint16_t* __restrict__ out, int H, int R, int n_parts,
+                                                            int part) {
+  const int row = blockIdx.x / H, head = blockIdx.x - row * H;
+  const size_t rh = (size_t)row * H + head;
+  const int np = min(n_parts, positions[row] / part + 1);
+  float mx = -INFINITY;
+  for (int p = 0; p < np; ++p) mx = fmaxf(mx, part_ml[(rh * n_parts + p) * 2]);
+  float lsum = 0.f;
+  for (int p = 0; p < np; ++p) lsum += exp2f(part_ml[(rh * n_parts + p) * 2] - mx) * part_ml[(rh * n_parts + p) * 2 + 1];
+  const float g = 1.f / (1.f + expf(-gate[(size_t)row * ldg + head]));
+  for (int c = threadIdx.x; c < R; c += 128) {
+    float acc = 0.f;
+    for (int p = 0; p < np; ++p)
+      acc = fmaf(exp2f(part_ml[(rh * n_parts + p) * 2] - mx), part_o[(rh * n_parts + p) * R + c], acc);
+    out[rh * R + c] = f2bf(acc / lsum * g);
+  }
+}
+
+template <int NR>
+static int launch_lat(const LatArgs& a, int split, int mt2, int n_head_chunks, hipStream_t s) {
+  const dim3 grid((a.n_items + 3) / 4, split ? a.n_parts : 1, n_head_chunks);
+  if (split) {
+    hipLaunchKernelGGL((latent_attn_mfma_kernel<NR, 1, true>), grid, dim3(256), 0, s, a);
+  } else if (mt2) {
+    if constexpr (NR <= 8) hipLaunchKernelGGL((latent_attn_mfma_kernel<NR, 2, false>), grid, dim3(256), 0, s, a);
+    else return (int)hipErrorInvalidValue;
+  } else {
+    hipLaunchKernelGGL((latent_attn_mfma_kernel<NR, 1, false>), grid, dim3(256), 0, s, a);
+  }
+  return (int)hipGetLastError();
+}
+
+}  // namespace k8s
+
+// 1 when the MFMA kernels take latent rank R (tiles per wave for prompt portions: 2 up to R = 256).
+K8S_API int k8s_latent_attn_mfma_ok(int R) {
+  switch (R) {
+    case 32: case 64: case 96: case 128: case 192: case 256: case 384: case 512: return R <= 256 ? 2 : 1;
+    default: return 0;
+  }
+}
+
+// split = 1: decode rows (items of one token), partials + merge into out; `positions` [T] are the
+// rows' positions and n_rows the number of decode rows (the first rows of the step).
+// split = 0: prompt portions, items of up to tiles * (16 / min(H, 16)) tokens.
+K8S_API int k8s_latent_attn_mfma(const void* qa, const void* c, const void* ct, const int* bt, int maxb,
+                                 const int* items, int n_items, const float* gate, int ldg, void* out,
+                                 float* part_o, float* part_ml, int n_parts, int part, const int* positions,
+                                 int n_rows, int H, int R, int BS, float scale, int split, int tiles,
+                                 hipStream_t s) {
+  if (n_items <= 0) return 0;
+  if (!k8s_latent_attn_mfma_ok(R) || BS % 32 || H <= 0 || (split && part % 32)) return (int)hipErrorInvalidValue;
+  k8s::LatArgs a;
+  a.qa = (const uint16_t*)qa; a.c = (const uint16_t*)c; a.ct = (const uint16_t*)ct; a.bt = bt; a.maxb = maxb;
+  a.items = items; a.n_items = n_items; a.gate = gate; a.ldg = ldg; a.out = (uint16_t*)out;
+  a.part_o = part_o; a.part_ml = part_ml; a.n_parts = n_parts; a.part = part;
+  a.H = H; a.HC = H < 16 ? H : 16; a.TPM = 16 / a.HC; a.BS = BS; a.scale_log2 = scale * k8s::kLog2e;
+  const int nhc = (H + a.HC - 1) / a.HC, mt2 = (!split && tiles == 2);
+  int rc;
+  switch (R / 32) {
+    case 1: rc = k8s::launch_lat<1>(a, split, mt2, nhc, s); break;
+    case 2: rc = k8s::launch_lat<2>(a, split, mt2, nhc, s); break;
+    case 3: rc = k8s::launch_lat<3>(a, split, mt2, nhc, s); break;
+    case 4: rc = k8s::launch_lat<4>(a, split, mt2, nhc, s); break;
+    case 6: rc = k8s::launch_lat<6>(a, split, mt2, nhc, s); break;
+    case 8: rc = k8s::launch_lat<8>(a, split, mt2, nhc, s); break;
+    case 12: rc = k8s::launch_lat<12>(a, split, mt2, nhc, s); break;
+    case 16: rc = k8s::launch_lat<16>(a, split, mt2, nhc, s); break;
+    default: return (int)hipErrorInvalidValue;
+  }
+  if (rc || !split) return rc;
+  hipLaunchKernelGGL(k8s::latent_reduce_kernel, dim3(n_rows * H), dim3(128), 0, s, part_o, part_ml, positions, gate, ldg,
+                     (uint16_t*)out, H, R, n_parts, part);
+  return (int)hipGetLastError();
+}

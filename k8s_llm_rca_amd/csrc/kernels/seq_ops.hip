@@ -169,12 +169,14 @@ __global__ void __launch_bounds__(256) postnorm_kernel(float* __restrict__ x, co
 // One row of the joint down projection [T][ld] fp32 = (query latent | key-value
 // latent): both are divided by their root mean square and scaled by a plain
 // weight.  The query latent goes to cq [T][QR]; the key-value latent (KR > 0)
-// to the paged latent cache at slots[t] (skipped when negative).
+// to the paged latent cache at slots[t] (skipped when negative), and to its
+// transposed twin cache_t when there is one.
 template <typename TW, typename TA>
 __global__ void __launch_bounds__(256) latent_norm_kernel(const float* __restrict__ dn, int ld,
                                                           const TW* __restrict__ wq, const TW* __restrict__ wkv,
                                                           const int* __restrict__ slots, TA* __restrict__ cq,
-                                                          TA* __restrict__ cache, int QR, int KR, float eps) {
+                                                          TA* __restrict__ cache, TA* __restrict__ cache_t, int BS,
+                                                          int QR, int KR, float eps) {
   __shared__ float scratch[16];
   const int t = blockIdx.x;
   const float* row = dn + (size_t)t * ld;
@@ -190,7 +192,12 @@ __global__ void __launch_bounds__(256) latent_norm_kernel(const float* __restric
   ss = block_sum(ss, scratch);
   inv = 1.f / sqrtf(ss / (float)KR + eps);
   if (slot < 0) return;
-  for (int c = threadIdx.x; c < KR; c += 256) stf(cache, (size_t)slot * KR + c, row[QR + c] * inv * ldf(wkv, c));
+  const size_t page = slot / BS, off = slot - page * BS;
+  for (int c = threadIdx.x; c < KR; c += 256) {
+    const float v = row[QR + c] * inv * ldf(wkv, c);
+    stf(cache, (size_t)slot * KR + c, v);
+    if (cache_t) stf(cache_t, (page * KR + c) * BS + off, v);   // the transposed pages [pages][KR][BS]
+  }
 }
 
 }  // namespace k8s
@@ -261,9 +268,10 @@ K8S_API int k8s_postnorm(float* x, const void* y, int y_dt, const void* w, int w
 }
 
 K8S_API int k8s_latent_norm(const float* dn, int ld, const void* wq, const void* wkv, const int* slots, void* cq,
-                            void* cache, int T, int QR, int KR, float eps, int dt, hipStream_t s) {
+                            void* cache, void* cache_t, int BS, int T, int QR, int KR, float eps, int dt,
+                            hipStream_t s) {
   if (T <= 0) return 0;
   K8S_DT2(dt, hipLaunchKernelGGL((latent_norm_kernel<TW, TA>), dim3(T), dim3(256), 0, s, dn, ld, (const TW*)wq,
-                                  (const TW*)wkv, slots, (TA*)cq, (TA*)cache, QR, KR, eps));
+                                  (const TW*)wkv, slots, (TA*)cq, (TA*)cache, (TA*)cache_t, BS, QR, KR, eps));
   return (int)hipGetLastError();
 }

@@ -139,19 +139,27 @@ class KVPool:
 class LatentKVPool(KVPool):
     """The same page allocator over LATENT pages: one tensor ``c[i]`` of shape
     ``[num_blocks, block_size, ranks[i]]`` per layer that projects its own
-    key-value latent (layers that attend over another layer's latents hold none).
-    A page index means the same token range in every tensor."""
+    key-value latent (layers that attend over another layer's latents hold none),
+    plus its transposed twin ``ct[i]`` ``[num_blocks, ranks[i], block_size]`` where
+    the MFMA attention kernels take that rank.  A page index means the same token
+    range in every tensor."""
 
     def __init__(self, ranks: List[int], num_blocks: int, block_size: int, device, dtype=torch.bfloat16):
         self.ranks = list(ranks)
         super().__init__(len(ranks), 1, max(ranks) if ranks else 0, num_blocks, block_size, device, dtype)
 
     def _alloc_storage(self, device, dtype) -> None:
+        from ..ops.seq_ops import mfma_tiles
         self.k = self.v = None
-        self.c = [torch.zeros(self.num_blocks, self.block_size, r, dtype=dtype, device=device) for r in self.ranks]
+        nb, BS = self.num_blocks, self.block_size
+        # zero-filled: a masked key of a stale page multiplies its value by 0, which must stay finite
+        self.c = [torch.zeros(nb, BS, r, dtype=dtype, device=device) for r in self.ranks]
+        # transposed twins [pages, rank, BS] where the MFMA attention kernels run (their PV operand)
+        self.ct = [torch.zeros(nb, r, BS, dtype=dtype, device=device) if mfma_tiles(r, dtype, device) else None
+                   for r in self.ranks]
 
     def tensors(self) -> tuple:
-        return (self.c,)
+        return (self.c, self.ct)
 
 
 class StatePool:

@@ -223,7 +223,9 @@ class ZasapelModel:
 
     # ------------------------------------------------------- what the engine allocates for this model
     def cache_bytes_per_block(self, block_size: int) -> int:
-        return sum(self.cache_ranks) * block_size * (2 if self.dtype == torch.bfloat16 else 4)
+        twice = [2 if S.mfma_tiles(r, self.dtype, self.device) else 1 for r in self.cache_ranks]
+        return sum(r * t for r, t in zip(self.cache_ranks, twice)) * block_size * (2 if self.dtype == torch.bfloat16
+                                                                                    else 4)
 
     def make_cache(self, num_blocks: int, block_size: int):
         from ..engine.kv_cache import LatentKVPool
@@ -279,6 +281,8 @@ class ZasapelModel:
                 L["w_uq"] = put(p + "mix.uq")
                 # absorbed forms: per head [D, KR] (fp32: the query is moved into latent space exactly) and [KR, V]
                 L["uk"] = put(p + "mix.uk", dtype=torch.float32).view(H, D, KR).contiguous()
+                if S.mfma_tiles(KR, dt, dev):
+                    L["uk16"] = put(p + "mix.uk").view(H, D, KR).contiguous()
                 L["uv_t"] = put(p + "mix.uv").view(H, V, KR).transpose(1, 2).contiguous()
                 L["wo"] = put(p + "mix.o")
             if ff is not None:
@@ -307,20 +311,25 @@ class ZasapelModel:
         y = S.mingru_scan(zug, L["bz"], L["bu"], states[f"gru{self.gru_of[li]}"], seg, self.dtype)
         return self._lin32(y, L["wo"])
 
-    def _latent_attention(self, li: int, h: torch.Tensor, inp: SegStepInputs, caches) -> torch.Tensor:
+    def _latent_attention(self, li: int, h: torch.Tensor, inp: SegStepInputs, caches, caches_t) -> torch.Tensor:
         L = self.layers[li]
         mx = self.cfg.layers[li][0]
         H, D, V, QR, KR = mx.heads, mx.dim, mx.vdim, mx.q_rank, mx.kv_rank
         T = h.shape[0]
-        cache = caches[self.cache_of[li]]
+        cache, cache_t = caches[self.cache_of[li]], caches_t[self.cache_of[li]]
         own = mx.kv_from is None
         dn = self._lin32(h, L["w_in"])                       # [T, QR (+ KR) + H] fp32: latents and gate logits
         cq = S.latent_norm(dn, L["dq_norm"], L["dkv_norm"] if own else None, inp.slots, cache if own else None,
-                           QR, KR, self.cfg.rms_eps, self.dtype)
+                           QR, KR, self.cfg.rms_eps, self.dtype, cache_t=cache_t)
         q = linear(cq, L["w_uq"]).view(T, H, D)
-        qa = torch.bmm(q.float().transpose(0, 1), L["uk"]).transpose(0, 1).contiguous()   # [T, H, KR] fp32
         gate = dn[:, QR + (KR if own else 0):]
-        o_lat = S.latent_attention(qa, cache, gate, inp.seg, mx.scale, self.dtype)        # [T, H, KR], gated
+        if cache_t is not None:
+            # matrix cores: the query moves into latent space as a bf16 batched product (fp32 accumulation)
+            qa = torch.bmm(q.transpose(0, 1), L["uk16"]).transpose(0, 1).contiguous()     # [T, H, KR] bf16
+            o_lat = S.latent_attention_mfma(qa, cache, cache_t, gate, inp.seg, inp.positions, mx.scale)
+        else:
+            qa = torch.bmm(q.float().transpose(0, 1), L["uk"]).transpose(0, 1).contiguous()   # [T, H, KR] fp32
+            o_lat = S.latent_attention(qa, cache, gate, inp.seg, mx.scale, self.dtype)    # [T, H, KR], gated
         o = torch.bmm(o_lat.transpose(0, 1), L["uv_t"]).transpose(0, 1).reshape(T, H * V)
         return self._lin32(o, L["wo"])
 
@@ -341,10 +350,11 @@ class ZasapelModel:
         yp = M.grouped_gemm(act, L["w2"], offsets)
         return M.combine_f32(yp, inv, T, ff.top)
 
-    def forward(self, inp: SegStepInputs, caches: List[torch.Tensor], states: Dict[str, torch.Tensor],
-                layers_out: Optional[list] = None) -> torch.Tensor:
+    def forward(self, inp: SegStepInputs, caches: List[torch.Tensor], caches_t: List[Optional[torch.Tensor]],
+                states: Dict[str, torch.Tensor], layers_out: Optional[list] = None) -> torch.Tensor:
         """Logits [len(logits_idx), vocab] fp32.  ``caches``: one paged latent tensor per layer with its own
-        key-value projection; ``states``: the per-slot tensors of :meth:`state_spec`.  ``layers_out``
+        key-value projection (``caches_t``: their transposed twins, or None); ``states``: the per-slot
+        tensors of :meth:`state_spec`.  ``layers_out``
         (debugging): receives a copy of the residual after every layer."""
         cfg = self.cfg
         seg = inp.seg
@@ -352,7 +362,8 @@ class ZasapelModel:
         for li, ((mx, ff), L) in enumerate(zip(cfg.layers, self.layers)):
             c1, c2 = self.conv_of[li]
             h = S.canon_conv(x, L["canon1"], states[f"conv{c1}"], seg, self.dtype)
-            y = self._mingru(li, h, seg, states) if mx.kind == "mingru" else self._latent_attention(li, h, inp, caches)
+            y = self._mingru(li, h, seg, states) if mx.kind == "mingru" else self._latent_attention(li, h, inp, caches,
+                                                                                                      caches_t)
             S.postnorm_(x, y, L["norm1"], cfg.postln_alpha, cfg.rms_eps)
             if ff is not None:
                 h = S.canon_conv(x, L["canon2"], states[f"conv{c2}"], seg, self.dtype)

@@ -11,12 +11,16 @@ the activation / weight type (bf16 or fp32).
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
-from typing import List, Optional
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Tuple
+
+import numpy as np
 
 import torch
 
-from ._lib import check, lib, ptr, stream_ptr, use_hip
+from ._lib import check, lib, ptr, scratch, stream_ptr, use_hip
+
+DECODE_PART = 256   # keys per partition of a decode row (split-KV); borders depend on the key index only
 
 
 @dataclass
@@ -30,8 +34,33 @@ class SegMeta:
     row0_host: List[int]
     pos0_host: List[int]
     slot_host: List[int]
-    # rows [0, n_single) are one-token segments (decode kernels); the rest portions of prompts
+    # rows [0, n_single) take the decode kernels (single tokens, short portions); the rest are prompt portions
     n_single: int = 0
+    _items: Dict[int, tuple] = field(default_factory=dict)
+
+    def attn_items(self, tokens_per_item: int) -> tuple:
+        """Work items of the MFMA attention kernels, made once per step and item size:
+        (decode items [n, 4] int32 on the device, prompt items, most keys a decode row sees).
+        An item is (segment, first row, tokens, position of the first row's token)."""
+        got = self._items.get(tokens_per_item)
+        if got is not None:
+            return got
+        dec, pre, kmax = [], [], 0
+        for s in range(self.n_seg):
+            a, b, p0 = self.row0_host[s], self.row0_host[s + 1], self.pos0_host[s]
+            if a < self.n_single:
+                dec += [(s, r, 1, p0 + r - a) for r in range(a, b)]
+                kmax = max(kmax, p0 + b - a)
+            else:
+                pre += [(s, r, min(tokens_per_item, b - r), p0 + r - a) for r in range(a, b, tokens_per_item)]
+        host = torch.from_numpy(np.asarray(dec + pre, dtype=np.int32).reshape(-1, 4))
+        dev = self.row_seg.device
+        if dev.type == "cuda":
+            host = host.pin_memory()
+        both = host.to(dev, non_blocking=True)
+        got = (both[:len(dec)], both[len(dec):], kmax)
+        self._items[tokens_per_item] = got
+        return got
 
 
 def _dt(t: torch.dtype) -> int:
@@ -140,18 +169,23 @@ def unit_norm_out(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
 
 
 def latent_norm(dn: torch.Tensor, wq: torch.Tensor, wkv: Optional[torch.Tensor], slots: torch.Tensor,
-                cache: Optional[torch.Tensor], q_rank: int, kv_rank: int, eps: float, out_dtype) -> torch.Tensor:
+                cache: Optional[torch.Tensor], q_rank: int, kv_rank: int, eps: float, out_dtype,
+                cache_t: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Rows of the joint down projection ``dn`` [T, >= q_rank + kv_rank] fp32: the query latent is
     RMS-normed (plain weight) and returned; the key-value latent (``wkv`` given) is RMS-normed and
-    written to the paged latent ``cache`` [pages, BS, kv_rank] at ``slots`` (page * BS + offset)."""
+    written to the paged latent ``cache`` [pages, BS, kv_rank] at ``slots`` (page * BS + offset), and
+    to its transposed twin ``cache_t`` [pages, kv_rank, BS] when given (the MFMA kernels' PV operand)."""
     T = dn.shape[0]
     cq = torch.empty(T, q_rank, dtype=out_dtype, device=dn.device)
     kr = kv_rank if wkv is not None else 0
     if use_hip(dn):
         assert dn.dtype == torch.float32 and dn.stride(1) == 1 and wq.dtype == out_dtype
         assert cache is None or (cache.is_contiguous() and cache.dtype == out_dtype and cache.shape[-1] == kv_rank)
-        check(lib().k8s_latent_norm(ptr(dn), dn.stride(0), ptr(wq), ptr(wkv), ptr(slots), ptr(cq), ptr(cache), T,
-                                    q_rank, kr, float(eps), _dt(out_dtype), stream_ptr(dn)), "latent_norm")
+        ct = cache_t if kr else None
+        assert ct is None or (ct.is_contiguous() and ct.dtype == out_dtype and ct.shape[1] == kv_rank)
+        check(lib().k8s_latent_norm(ptr(dn), dn.stride(0), ptr(wq), ptr(wkv), ptr(slots), ptr(cq), ptr(cache),
+                                    ptr(ct), cache.shape[1] if kr else 1, T, q_rank, kr, float(eps),
+                                    _dt(out_dtype), stream_ptr(dn)), "latent_norm")
         return cq
     q = dn[:, :q_rank]
     cq.copy_((q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * wq.float()).to(out_dtype))
@@ -160,7 +194,50 @@ def latent_norm(dn: torch.Tensor, wq: torch.Tensor, wkv: Optional[torch.Tensor],
         c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * wkv.float()
         ok = slots >= 0
         cache.view(-1, kr)[slots[ok].long()] = c[ok].to(cache.dtype)
+        if cache_t is not None:
+            BS = cache.shape[1]
+            sl = slots[ok].long()
+            cache_t[sl // BS, :, sl % BS] = c[ok].to(cache_t.dtype)
     return cq
+
+
+def mfma_tiles(R: int, dtype, device) -> int:
+    """Query tiles per wave the MFMA attention kernels run prompt portions with for latent rank ``R``
+    (0: they do not take this rank or type -- the vector-pipe kernel runs instead)."""
+    if dtype != torch.bfloat16 or torch.device(device).type != "cuda":
+        return 0
+    return int(lib().k8s_latent_attn_mfma_ok(int(R)))
+
+
+def latent_attention_mfma(qa: torch.Tensor, cache: torch.Tensor, cache_t: torch.Tensor, gate: torch.Tensor,
+                          seg: SegMeta, positions: torch.Tensor, scale: float) -> torch.Tensor:
+    """:func:`latent_attention` on the matrix cores: bf16 absorbed queries ``qa`` [T, H, R], the latent
+    pages and their transposed twins.  Decode rows (the step's first ``seg.n_single``) are split over
+    partitions of ``DECODE_PART`` keys and merged; prompt portions run one wave per group of tokens."""
+    T, H, R = qa.shape
+    BS = cache.shape[1]
+    tiles = mfma_tiles(R, qa.dtype, qa.device)
+    assert tiles and qa.is_contiguous() and cache.is_contiguous() and cache_t.is_contiguous() and BS % 32 == 0
+    assert gate.dtype == torch.float32 and gate.stride(1) == 1 and seg.block_tables.is_contiguous()
+    out = torch.empty(T, H, R, dtype=torch.bfloat16, device=qa.device)
+    tpi = tiles * (16 // min(H, 16))
+    dec, pre, kmax = seg.attn_items(tpi)
+    L, st = lib(), stream_ptr(qa)
+    bt, maxb = seg.block_tables, seg.block_tables.shape[1]
+    if dec.shape[0]:
+        n_parts = -(-kmax // DECODE_PART)
+        nd = seg.n_single
+        part_o = scratch(nd * H * n_parts * R, torch.float32, qa.device)
+        part_ml = scratch(nd * H * n_parts * 2, torch.float32, qa.device)
+        check(L.k8s_latent_attn_mfma(ptr(qa), ptr(cache), ptr(cache_t), ptr(bt), maxb, ptr(dec), dec.shape[0],
+                                     ptr(gate), gate.stride(0), ptr(out), ptr(part_o), ptr(part_ml), n_parts,
+                                     DECODE_PART, ptr(positions), nd, H, R, BS, float(scale), 1, 1, st),
+              "latent_attn_mfma (decode)")
+    if pre.shape[0]:
+        check(L.k8s_latent_attn_mfma(ptr(qa), ptr(cache), ptr(cache_t), ptr(bt), maxb, ptr(pre), pre.shape[0],
+                                     ptr(gate), gate.stride(0), ptr(out), None, None, 1, DECODE_PART, None, 0,
+                                     H, R, BS, float(scale), 0, tiles, st), "latent_attn_mfma (prefill)")
+    return out
 
 
 def latent_attention(qa: torch.Tensor, cache: torch.Tensor, gate: torch.Tensor, seg: SegMeta, scale: float,

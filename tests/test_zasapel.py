@@ -129,8 +129,8 @@ def engine(d, W, backend, num_blocks=24, block_size=32, slots=4, **kw):
     eng = LLMEngine(EngineConfig(**cfg), model=model)
     for t in eng.states.t.values():       # a fresh slot must not be read: make a read loud
         t.fill_(float("nan"))
-    for c in eng.kv.c:
-        c.fill_(float("nan"))
+    for c in eng.kv.c + [t for t in eng.kv.ct if t is not None]:
+        c.fill_(3e4)                      # stale pages hold finite garbage (masked keys multiply it by 0)
     return eng
 
 
@@ -275,6 +275,66 @@ def test_latent_attention_finds_one_far_key(backend):
             o = S.latent_attention(qa[:1].to(dev).contiguous(), cache, gate[:1].to(dev), seg, 1.0, dt).float().cpu()
             hit = torch.allclose(o[0, 0], c[far], atol=2e-2)
             assert hit == (r >= far), (far, r)
+
+
+@GPU
+@pytest.mark.parametrize("H,R", [(1, 32), (3, 64), (16, 96), (20, 256), (8, 512), (5, 128)])
+def test_latent_attention_matrix_core_kernels(H, R):
+    """The MFMA kernels: prompt portions (one and two tiles per wave, heads fewer and more than a
+    tile), decode rows over several key partitions, pages in any order, stale pages behind the end."""
+    dev, dt = "cuda", torch.bfloat16
+    g = torch.Generator().manual_seed(H * 1000 + R)
+    n, BS = 700, 64
+    c = torch.randn(n, R, generator=g).to(dt).float()
+    qa = (torch.randn(n, H, R, generator=g) * 0.5).to(dt).float()
+    gate = torch.randn(n, H + 1, generator=g)
+    scale = 2.0 / math.sqrt(R)
+    sc = torch.einsum("thr,jr->thj", qa.double(), c.double()) * scale
+    sc = sc.masked_fill(torch.arange(n)[None, None, :] > torch.arange(n)[:, None, None], float("-inf"))
+    want = torch.einsum("thj,jr->thr", torch.softmax(sc, -1), c.double()) * torch.sigmoid(gate[:, :H].double())[..., None]
+    order = [7, 2, 11, 0, 5, 9, 3, 1, 10, 4, 8]
+    cache = torch.full((13, BS, R), 3e4, dtype=dt, device=dev)
+    cache_t = torch.full((13, R, BS), 3e4, dtype=dt, device=dev)
+    for j in range(n):
+        cache[order[j // BS], j % BS] = c[j].to(dt)
+        cache_t[order[j // BS], :, j % BS] = c[j].to(dt)
+    pos = torch.arange(n, dtype=torch.int32, device=dev)
+    outs = []
+    # a long portion, a short one, then decode rows: three at once (one sequence's consecutive tokens), then single
+    cuts = [(0, 300), (300, 303), (303, 650), (650, 653)] + [(i, i + 1) for i in range(653, n)]
+    for a, b in cuts:
+        seg = seg_meta([b - a], [a], [0], dev, [order])
+        seg.n_single = (b - a) if b - a <= 3 and a >= 650 else 0
+        outs.append(S.latent_attention_mfma(qa[a:b].to(dev, dt).contiguous(), cache, cache_t, gate[a:b].to(dev), seg,
+                                            pos[a:b].contiguous(), scale))
+    assert rel_err(torch.cat(outs).float().flatten(1), want.float().flatten(1)) < 2e-2
+
+
+@GPU
+def test_latent_attention_matrix_cores_find_one_far_key():
+    dev, dt = "cuda", torch.bfloat16
+    n, R, BS, H = 900, 64, 32, 4
+    for far in (0, 31, 32, 255, 256, 257, 511, 512, 640, n - 2):
+        c = torch.randn(n, R, generator=torch.Generator().manual_seed(far)).to(dt).float()
+        c[:, 0] = -c[:, 0].abs()
+        c[far] = 0
+        c[far, 0] = 8.0
+        qa = torch.zeros(1, H, R)
+        qa[:, :, 0] = 6.0
+        pages = list(range(29, -1, -1))
+        cache = torch.full((31, BS, R), 3e4, dtype=dt, device=dev)
+        cache_t = torch.full((31, R, BS), 3e4, dtype=dt, device=dev)
+        for j in range(n):
+            cache[pages[j // BS], j % BS] = c[j].to(dt)
+            cache_t[pages[j // BS], :, j % BS] = c[j].to(dt)
+        gate = torch.full((1, H), 30.0, device=dev)
+        for r in [n - 1] + ([far - 1] if far > 0 else []):
+            for single in (0, 1):                     # as a prompt row and as a decode row
+                seg = seg_meta([1], [r], [0], dev, [pages])
+                seg.n_single = single
+                o = S.latent_attention_mfma(qa.to(dev, dt), cache, cache_t, gate, seg,
+                                            torch.tensor([r], dtype=torch.int32, device=dev), 1.0).float().cpu()
+                assert torch.allclose(o[0, 0], c[far], atol=3e-2) == (r >= far), (far, r, single)
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
@@ -424,6 +484,20 @@ def test_page_borders_and_far_keys_sharp_softmax(backend):
     else:
         e = (got.double().cpu() - want.double()).pow(2).mean(-1).sqrt() / want.double().pow(2).mean(-1).sqrt()
         assert float(e.median()) < 0.05 and float(e.max()) < 0.5
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_decode_past_the_key_partition_border(backend):
+    """Decoded tokens whose keys span more than one split-KV partition (256 keys), rank 64 (matrix cores in bf16)."""
+    d = config([(attn(heads=4, dim=16, vdim=8, q_rank=24, kv_rank=64), None),
+                (attn(heads=2, dim=16, vdim=8, q_rank=24, kv_rank=64, kv_from=0), dense(32))],
+               width=32, vocab=128, taps=2)
+    W = weights(d, 22)
+    t = toks(270, d["vocab"], 23)
+    want = O.forward(d, W, t).float()
+    eng = engine(d, W, backend, num_blocks=6, block_size=64)
+    got = feed_all(eng, eng.new_sequence(), t, (250,))      # then 20 tokens one by one over key 256
+    assert rel_err(got, want) < tol(backend[1])
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
