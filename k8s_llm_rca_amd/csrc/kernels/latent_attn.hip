@@ -201,7 +201,11 @@ template <int NR, int MT, bool SPLIT>
 __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(LatArgs a) {
   constexpr int R = NR * 32, ND = R / 16;
   const int lane = threadIdx.x & 63, r = lane & 15, h = lane >> 4;
-  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+  // workgroups go round-robin over the 8 XCDs, each with its own L2: give every XCD a contiguous
+  // range of items (neighbouring token groups of the same sequences read the same latent pages)
+  const int per = gridDim.x >> 3;
+  const int blk = (gridDim.x & 7) == 0 ? (blockIdx.x & 7) * per + (blockIdx.x >> 3) : blockIdx.x;
+  const int item = blk * 4 + (threadIdx.x >> 6);
   if (item >= a.n_items) return;
   const int sg = a.items[item * 4], row0 = a.items[item * 4 + 1], ntok = a.items[item * 4 + 2],
             pos0 = a.items[item * 4 + 3];
@@ -324,6 +328,165 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(LatArgs a) {
   }
 }
 
+// Prompt portions: the four waves of a workgroup own four consecutive items of ONE
+// segment (the host pads every segment's items to a multiple of four with empty
+// ones), so they read the same keys.  A chunk's operand fragments do not depend on
+// the item: kf[t][cc] and vf[dt] are loaded from global memory once per workgroup
+// (a quarter by each wave), parked in LDS in fragment order -- slot f holds the 64
+// lanes' 16 bytes, so writes and reads are conflict-free -- and read back by all
+// four waves.  Two buffers: chunk i + 1 is fetched into registers while chunk i
+// is computed, and written after it; one barrier per chunk.
+template <int NR, int MT>
+__global__ void __launch_bounds__(256) latent_attn_mfma_lds_kernel(LatArgs a) {
+  constexpr int R = NR * 32, ND = R / 16, NF = 2 * NR + ND, NFW = NF / 4;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  bf16x8* frag = reinterpret_cast<bf16x8*>(lds_raw);          // [2][NF][64]
+  __shared__ int kend_s[4];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, r = lane & 15, h = lane >> 4;
+  const int per = gridDim.x >> 3;
+  const int blk = (gridDim.x & 7) == 0 ? (blockIdx.x & 7) * per + (blockIdx.x >> 3) : blockIdx.x;
+  const int item0 = blk * 4;
+  if (item0 >= a.n_items) return;                              // whole workgroup
+  const int item = item0 + wv;
+  const int sg = a.items[item0 * 4];
+  const int row0 = a.items[item * 4 + 1], ntok = a.items[item * 4 + 2], pos0 = a.items[item * 4 + 3];
+  const int hc = blockIdx.z;
+  if (lane == 0) kend_s[wv] = ntok > 0 ? pos0 + ntok : 0;
+  __syncthreads();
+  const int k_end = max(max(kend_s[0], kend_s[1]), max(kend_s[2], kend_s[3]));
+  const int tl = r / a.HC, hl = r - tl * a.HC, head = hc * a.HC + hl;
+  bf16x8 qf[MT][NR];
+  int limit[MT];
+  f32x4 o[MT][ND];
+  float m[MT], l[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int ti = mt * a.TPM + tl;
+    const bool valid = tl < a.TPM && ti < ntok && head < a.H;
+    limit[mt] = valid ? pos0 + ti + 1 : 0;
+    const uint16_t* qp = a.qa + ((size_t)(row0 + (valid ? ti : 0)) * a.H + (valid ? head : 0)) * R;
+#pragma unroll
+    for (int cc = 0; cc < NR; ++cc) {
+      qf[mt][cc] = ld16(qp + 32 * cc + 8 * h);
+      if (!valid)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) qf[mt][cc][j] = (__bf16)0.f;
+    }
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt) o[mt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m[mt] = -INFINITY;
+    l[mt] = 0.f;
+  }
+  const int* pages = a.bt + (size_t)sg * a.maxb;
+  // this wave's share of a chunk's fragments: f = wv + 4 i
+  bf16x8 pre[NFW];
+  auto fetch = [&](int kb) {
+    const int page = pages[kb / a.BS], off = kb % a.BS;
+    const uint16_t* cp = a.c + (size_t)page * a.BS * R;
+    const uint16_t* tp = a.ct + (size_t)page * R * a.BS;
+#pragma unroll
+    for (int i = 0; i < NFW; ++i) {
+      const int f = wv + 4 * i;
+      if (f < 2 * NR) {
+        const int t = f / NR, cc = f - t * NR;
+        const int key = off + 8 * (r >> 2) + 4 * t + (r & 3);
+        pre[i] = ld16(cp + (size_t)key * R + 32 * cc + 8 * h);
+      } else {
+        const int dt = f - 2 * NR;
+        pre[i] = ld16(tp + (size_t)(16 * dt + r) * a.BS + off + 8 * h);
+      }
+    }
+  };
+  auto park = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < NFW; ++i) frag[((size_t)buf * NF + wv + 4 * i) * 64 + lane] = pre[i];
+  };
+  if (k_end > 0) {
+    fetch(0);
+    park(0);
+  }
+  int buf = 0;
+  for (int kb = 0; kb < k_end; kb += 32, buf ^= 1) {
+    __syncthreads();
+    const bool more = kb + 32 < k_end;
+    if (more) fetch(kb + 32);
+    const bf16x8* fb = frag + (size_t)buf * NF * 64 + lane;
+    f32x4 s[MT][2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) s[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int cc = 0; cc < NR; ++cc) {
+        const bf16x8 kf = fb[(t * NR + cc) * 64];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          s[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[mt][cc], s[mt][t], 0, 0, 0);
+      }
+    }
+    bf16x8 pf[MT];
+    float ar[MT][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      float p[8];
+      float cmax = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = kb + 8 * h + 4 * t + i;
+          const float v = key < limit[mt] ? s[mt][t][i] * a.scale_log2 : -INFINITY;
+          p[4 * t + i] = v;
+          cmax = fmaxf(cmax, v);
+        }
+      cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
+      cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
+      const float mnew = fmaxf(m[mt], cmax);
+      const float alpha = (mnew == -INFINITY) ? 1.f : exp2f(m[mt] - mnew);
+      float psum = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float e = (mnew == -INFINITY) ? 0.f : exp2f(p[j] - mnew);
+        psum += e;
+        pf[mt][j] = (__bf16)e;
+      }
+      l[mt] = l[mt] * alpha + psum;
+      m[mt] = mnew;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ar[mt][i] = __shfl(alpha, 4 * h + i, 64);
+    }
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt) {
+      const bf16x8 vf = fb[(2 * NR + dt) * 64];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[mt][dt][i] *= ar[mt][i];
+        o[mt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf[mt], vf, o[mt][dt], 0, 0, 0);
+      }
+    }
+    if (more) park(buf ^ 1);
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    float lt = l[mt];
+    lt += __shfl_xor(lt, 16, 64);
+    lt += __shfl_xor(lt, 32, 64);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int q = 4 * h + i;
+      const int qtl = q / a.HC, qhl = q - qtl * a.HC, qhead = hc * a.HC + qhl, ti = mt * a.TPM + qtl;
+      const float lq = __shfl(lt, q, 64);
+      if (!(qtl < a.TPM && ti < ntok && qhead < a.H)) continue;
+      const size_t rh = (size_t)(row0 + ti) * a.H + qhead;
+      const float g = 1.f / (1.f + expf(-a.gate[(size_t)(row0 + ti) * a.ldg + qhead]));
+      const float sc = lq > 0.f ? g / lq : 0.f;
+#pragma unroll
+      for (int dt = 0; dt < ND; ++dt) a.out[rh * R + 16 * dt + r] = f2bf(o[mt][dt][i] * sc);
+    }
+  }
+}
+
 // Merge of the key partitions of decode rows: one workgroup per (row, head).
 // A row at position p has ceil((p + 1) / part) partitions.
 __global__ void __launch_bounds__(128) latent_reduce_kernel(const float* __restrict__ part_o,
@@ -350,15 +513,28 @@ __global__ void __launch_bounds__(128) latent_reduce_kernel(const float* __restr
 
 template <int NR>
 static int launch_lat(const LatArgs& a, int split, int mt2, int n_head_chunks, hipStream_t s) {
-  const dim3 grid((a.n_items + 3) / 4, split ? a.n_parts : 1, n_head_chunks);
+  int nblk = (a.n_items + 3) / 4;
+  if (nblk > 8) nblk = (nblk + 7) & ~7;   // a multiple of the XCD count (the kernels' item remap)
+  const dim3 grid(nblk, split ? a.n_parts : 1, n_head_chunks);
   if (split) {
     hipLaunchKernelGGL((latent_attn_mfma_kernel<NR, 1, true>), grid, dim3(256), 0, s, a);
-  } else if (mt2) {
-    if constexpr (NR <= 8) hipLaunchKernelGGL((latent_attn_mfma_kernel<NR, 2, false>), grid, dim3(256), 0, s, a);
-    else return (int)hipErrorInvalidValue;
-  } else {
-    hipLaunchKernelGGL((latent_attn_mfma_kernel<NR, 1, false>), grid, dim3(256), 0, s, a);
+    return (int)hipGetLastError();
   }
+  if (a.n_items % 4) return (int)hipErrorInvalidValue;   // prompt items come in fours per segment
+  constexpr size_t lds = 2 * (size_t)(4 * NR) * 64 * 16;  // two buffers of 2 NR + R / 16 fragments of 1 KiB
+  if constexpr (NR <= 8) {
+    if (mt2) {
+      auto k = latent_attn_mfma_lds_kernel<NR, 2>;
+      if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
+        return (int)hipGetLastError();
+      hipLaunchKernelGGL(k, grid, dim3(256), lds, s, a);
+      return (int)hipGetLastError();
+    }
+  }
+  auto k = latent_attn_mfma_lds_kernel<NR, 1>;
+  if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
+    return (int)hipGetLastError();
+  hipLaunchKernelGGL(k, grid, dim3(256), lds, s, a);
   return (int)hipGetLastError();
 }
 

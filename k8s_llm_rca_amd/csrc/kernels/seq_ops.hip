@@ -141,6 +141,72 @@ __global__ void __launch_bounds__(256) mingru_scan_kernel(const float* __restric
   *st = S;
 }
 
+// The same recurrence for long segments, parallel over time: the rows are cut in
+// chunks ([n][4] int32: segment, first row, rows, index of the segment's first
+// chunk).  Pass 1 reduces every chunk to (A, B) with S_out = A S_in + B and saves
+// the segment's incoming state; pass 2 folds the earlier chunks' (A, B) into the
+// chunk's S_in, runs the chunk step by step as the sequential kernel does, and
+// the segment's last chunk stores the state.
+__device__ __forceinline__ void mingru_gates(const float* row, int C, int c, float vbz, float vbu, float& z,
+                                             float& cand) {
+  z = 1.f / (1.f + expf(-(row[c] + vbz)));
+  const float u = row[C + c] + vbu;
+  cand = u >= 0.f ? u + 0.5f : 1.f / (1.f + expf(-u));
+}
+
+template <typename TW>
+__global__ void __launch_bounds__(256) mingru_chunk_sum_kernel(const float* __restrict__ zug, const TW* __restrict__ bz,
+                                                               const TW* __restrict__ bu,
+                                                               const float* __restrict__ state,
+                                                               const int* __restrict__ chunks,
+                                                               const int* __restrict__ seg_pos0,
+                                                               const int* __restrict__ seg_slot,
+                                                               float* __restrict__ ab, float* __restrict__ s0, int C) {
+  const int ck = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int sg = chunks[ck * 4], r0 = chunks[ck * 4 + 1], n = chunks[ck * 4 + 2], first = chunks[ck * 4 + 3];
+  const float vbz = ldf(bz, c), vbu = ldf(bu, c);
+  float A = 1.f, B = 0.f;
+#pragma unroll 4
+  for (int r = r0; r < r0 + n; ++r) {
+    float z, cand;
+    mingru_gates(zug + (size_t)r * 3 * C, C, c, vbz, vbu, z, cand);
+    A *= 1.f - z;
+    B = (1.f - z) * B + z * cand;
+  }
+  ab[((size_t)ck * 2) * C + c] = A;
+  ab[((size_t)ck * 2 + 1) * C + c] = B;
+  if (ck == first) s0[(size_t)sg * C + c] = seg_pos0[sg] > 0 ? state[(size_t)seg_slot[sg] * C + c] : 0.f;
+}
+
+template <typename TW, typename TA>
+__global__ void __launch_bounds__(256) mingru_chunk_apply_kernel(const float* __restrict__ zug,
+                                                                 const TW* __restrict__ bz, const TW* __restrict__ bu,
+                                                                 float* __restrict__ state,
+                                                                 const int* __restrict__ chunks,
+                                                                 const int* __restrict__ seg_row0,
+                                                                 const int* __restrict__ seg_slot,
+                                                                 const float* __restrict__ ab,
+                                                                 const float* __restrict__ s0, TA* __restrict__ y,
+                                                                 int C) {
+  const int ck = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int sg = chunks[ck * 4], r0 = chunks[ck * 4 + 1], n = chunks[ck * 4 + 2], first = chunks[ck * 4 + 3];
+  float S = s0[(size_t)sg * C + c];
+  for (int j = first; j < ck; ++j) S = ab[((size_t)j * 2) * C + c] * S + ab[((size_t)j * 2 + 1) * C + c];
+  const float vbz = ldf(bz, c), vbu = ldf(bu, c);
+#pragma unroll 4
+  for (int r = r0; r < r0 + n; ++r) {
+    const float* row = zug + (size_t)r * 3 * C;
+    float z, cand;
+    mingru_gates(row, C, c, vbz, vbu, z, cand);
+    const float g = row[2 * C + c];
+    S = (1.f - z) * S + z * cand;
+    stf(y, (size_t)r * C + c, S * (g / (1.f + expf(-g))));
+  }
+  if (r0 + n == seg_row0[sg + 1]) state[(size_t)seg_slot[sg] * C + c] = S;
+}
+
 // x <- unit_rms(alpha x + y) * (1 + w), in place on the fp32 residual.
 // y == nullptr: x <- unit_rms(x) * (1 + w) into `out` (the model's last norm).
 template <typename TY, typename TW, typename TO>
@@ -244,6 +310,19 @@ K8S_API int k8s_mingru_scan(const float* zug, const void* bz, const void* bu, fl
   if (n_seg <= 0) return 0;
   K8S_DT2(dt, hipLaunchKernelGGL((mingru_scan_kernel<TW, TA>), dim3(n_seg, (C + 255) / 256), dim3(256), 0, s, zug,
                                   (const TW*)bz, (const TW*)bu, state, seg_row0, seg_pos0, seg_slot, (TA*)y, C));
+  return (int)hipGetLastError();
+}
+
+// ab: [n_chunks][2][C] fp32 scratch, s0: [n_seg][C] fp32 scratch.
+K8S_API int k8s_mingru_chunked(const float* zug, const void* bz, const void* bu, float* state, const int* chunks,
+                               int n_chunks, const int* seg_row0, const int* seg_pos0, const int* seg_slot,
+                               float* ab, float* s0, void* y, int C, int dt, hipStream_t s) {
+  if (n_chunks <= 0) return 0;
+  const dim3 grid(n_chunks, (C + 255) / 256);
+  K8S_DT2(dt, hipLaunchKernelGGL((mingru_chunk_sum_kernel<TW>), grid, dim3(256), 0, s, zug, (const TW*)bz,
+                                 (const TW*)bu, state, chunks, seg_pos0, seg_slot, ab, s0, C));
+  K8S_DT2(dt, hipLaunchKernelGGL((mingru_chunk_apply_kernel<TW, TA>), grid, dim3(256), 0, s, zug, (const TW*)bz,
+                                 (const TW*)bu, state, chunks, seg_row0, seg_slot, ab, s0, (TA*)y, C));
   return (int)hipGetLastError();
 }
 

@@ -345,9 +345,9 @@ class ZasapelModel:
         w, ids = M.route_direct(h, L["router"], ff.top, scoring="sigmoid", renorm=False)
         order, inv, offsets = M.align(ids, ff.experts)
         xp = M.gather_rows(h, order, ff.top, w)             # the weight multiplies the expert's input
-        gu = M.grouped_gemm(xp, L["w13"], offsets)
+        gu = M.grouped_auto(xp, L["w13"], offsets)
         act = M.glu_clamp(gu, GLU_ALPHA, ff.limit, GLU_UP_SHIFT)
-        yp = M.grouped_gemm(act, L["w2"], offsets)
+        yp = M.grouped_auto(act, L["w2"], offsets)
         return M.combine_f32(yp, inv, T, ff.top)
 
     def forward(self, inp: SegStepInputs, caches: List[torch.Tensor], caches_t: List[Optional[torch.Tensor]],

@@ -85,6 +85,7 @@ _SIGS = {
     "k8s_embed_sinpos": [P, P, P, P, I, I, F, I, P],
     "k8s_canon_conv": [P, P, P, P, P, P, P, P, I, I, I, I, I, P],
     "k8s_mingru_scan": [P, P, P, P, P, P, P, P, I, I, I, P],
+    "k8s_mingru_chunked": [P, P, P, P, P, I, P, P, P, P, P, P, I, I, P],
     "k8s_postnorm": [P, P, I, P, I, P, I, I, F, F, P],
     "k8s_latent_norm": [P, I, P, P, P, P, P, P, I, I, I, I, F, I, P],
     "k8s_latent_attn_mfma_ok": [I],

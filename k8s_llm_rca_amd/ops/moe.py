@@ -227,3 +227,17 @@ def combine_f32(y_perm: torch.Tensor, inv: torch.Tensor, T: int, k: int,
     if w is not None:
         g = g * w.view(T, k, 1)
     return g.sum(1)
+
+
+BIG_MIN_ROWS = 2048   # above: the prefill-size grouped GEMM (gemm_big.hip), as the Mixtral block picks it
+
+
+def grouped_auto(a: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor) -> torch.Tensor:
+    """``grouped_gemm`` with the kernel chosen by size: the grouped form of the prefill GEMM for
+    many rows, the weight-streaming grouped kernel for decode-size batches, the any-shape kernel
+    (or fp32) otherwise.  None of them reads the offsets on the host."""
+    E, N, K = w.shape
+    if (use_hip(a) and a.dtype == torch.bfloat16 and a.shape[0] > BIG_MIN_ROWS
+            and grouped_big_ok(a.shape[0], N, K, False)):
+        return grouped_big(a, w, offsets)
+    return grouped_gemm(a, w, offsets)

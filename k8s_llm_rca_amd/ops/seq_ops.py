@@ -41,7 +41,8 @@ class SegMeta:
     def attn_items(self, tokens_per_item: int) -> tuple:
         """Work items of the MFMA attention kernels, made once per step and item size:
         (decode items [n, 4] int32 on the device, prompt items, most keys a decode row sees).
-        An item is (segment, first row, tokens, position of the first row's token)."""
+        An item is (segment, first row, tokens, position of the first row's token); a segment's prompt
+        items are padded with empty ones to a multiple of four."""
         got = self._items.get(tokens_per_item)
         if got is not None:
             return got
@@ -53,6 +54,7 @@ class SegMeta:
                 kmax = max(kmax, p0 + b - a)
             else:
                 pre += [(s, r, min(tokens_per_item, b - r), p0 + r - a) for r in range(a, b, tokens_per_item)]
+                pre += [(s, a, 0, p0)] * (-len(pre) % 4)   # a workgroup's four waves share one segment's keys
         host = torch.from_numpy(np.asarray(dec + pre, dtype=np.int32).reshape(-1, 4))
         dev = self.row_seg.device
         if dev.type == "cuda":
@@ -61,6 +63,30 @@ class SegMeta:
         got = (both[:len(dec)], both[len(dec):], kmax)
         self._items[tokens_per_item] = got
         return got
+
+
+    def scan_chunks(self, rows: int) -> Optional[torch.Tensor]:
+        """Chunks of at most ``rows`` rows for the time-parallel recurrence ([n, 4] int32 on the device:
+        segment, first row, rows, index of the segment's first chunk); None when no segment is longer
+        than two chunks (the sequential kernel runs)."""
+        key = -rows
+        if key in self._items:
+            return self._items[key]
+        out = None
+        if max(b - a for a, b in zip(self.row0_host[:-1], self.row0_host[1:])) > 2 * rows:
+            ch = []
+            for s in range(self.n_seg):
+                a, b, first = self.row0_host[s], self.row0_host[s + 1], len(ch)
+                ch += [(s, r, min(rows, b - r), first) for r in range(a, b, rows)]
+            host = torch.from_numpy(np.asarray(ch, dtype=np.int32))
+            if self.row_seg.device.type == "cuda":
+                host = host.pin_memory()
+            out = host.to(self.row_seg.device, non_blocking=True)
+        self._items[key] = out
+        return out
+
+
+SCAN_CHUNK = 64     # rows per chunk of the time-parallel minGRU
 
 
 def _dt(t: torch.dtype) -> int:
@@ -124,6 +150,14 @@ def mingru_scan(zug: torch.Tensor, bz: torch.Tensor, bu: torch.Tensor, state: to
     y = torch.empty(T, C, dtype=out_dtype, device=zug.device)
     if use_hip(zug):
         assert zug.dtype == torch.float32 and zug.is_contiguous() and state.is_contiguous() and bz.dtype == out_dtype
+        chunks = seg.scan_chunks(SCAN_CHUNK)
+        if chunks is not None:   # long prompt portions: parallel over time as well as channels
+            ab = scratch(chunks.shape[0] * 2 * C, torch.float32, zug.device)
+            s0 = scratch(seg.n_seg * C, torch.float32, zug.device)
+            check(lib().k8s_mingru_chunked(ptr(zug), ptr(bz), ptr(bu), ptr(state), ptr(chunks), chunks.shape[0],
+                                           ptr(seg.seg_row0), ptr(seg.seg_pos0), ptr(seg.seg_slot), ptr(ab), ptr(s0),
+                                           ptr(y), C, _dt(out_dtype), stream_ptr(zug)), "mingru_chunked")
+            return y
         check(lib().k8s_mingru_scan(ptr(zug), ptr(bz), ptr(bu), ptr(state), ptr(seg.seg_row0), ptr(seg.seg_pos0),
                                     ptr(seg.seg_slot), ptr(y), seg.n_seg, C, _dt(out_dtype), stream_ptr(zug)),
               "mingru_scan")

@@ -223,6 +223,38 @@ def test_mingru_scan_matches_recurrence_across_portions(backend):
     assert rel_err(torch.cat(got).float(), want) < tol(dt)
 
 
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_mingru_long_portions_parallel_over_time(backend):
+    """Portions much longer than a scan chunk, two sequences in a step, continued afterwards."""
+    dev, dt = backend
+    g = torch.Generator().manual_seed(3)
+    C, na, nb = 70, 333, 200
+    bz, bu = torch.randn(C, generator=g).to(torch.bfloat16).float(), torch.randn(C, generator=g).to(torch.bfloat16).float()
+    za, zb = torch.randn(na, 3 * C, generator=g) * 1.5, torch.randn(nb, 3 * C, generator=g) * 1.5
+    wt = {"z": torch.eye(C), "x": torch.eye(C), "g": torch.eye(C), "z.b": bz, "x.b": bu, "o": torch.eye(C)}
+
+    def want(zug):
+        h = zug.double()
+        z = torch.sigmoid(h[:, :C] + bz.double())
+        u = h[:, C:2 * C] + bu.double()
+        cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+        S, ys = torch.zeros(C, dtype=torch.float64), []
+        for t in range(h.shape[0]):
+            S = (1 - z[t]) * S + z[t] * cand[t]
+            ys.append(S * torch.nn.functional.silu(h[t, 2 * C:]))
+        return torch.stack(ys).float()
+
+    state = torch.full((3, C), float("nan"), device=dev)
+    b_, u_ = bz.to(dev, dt), bu.to(dev, dt)
+    s1 = S.mingru_scan(torch.cat([za[:300], zb[:150]]).to(dev).contiguous(), b_, u_, state,
+                       seg_meta([300, 150], [0, 0], [2, 0], dev), dt)
+    s2 = S.mingru_scan(torch.cat([zb[150:], za[300:]]).to(dev).contiguous(), b_, u_, state,
+                       seg_meta([50, 33], [150, 300], [0, 2], dev), dt)
+    got_a = torch.cat([s1[:300], s2[50:]]).float()
+    got_b = torch.cat([s1[300:], s2[:50]]).float()
+    assert rel_err(got_a, want(za)) < tol(dt) and rel_err(got_b, want(zb)) < tol(dt)
+
+
 def paged(c, block_size, order, dev, dt):
     """Latents [n, R] scattered over pages in ``order``; returns (cache, block table row)."""
     n, R = c.shape
