@@ -336,15 +336,17 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(LatArgs a) {
 // lanes' 16 bytes, so writes and reads are conflict-free -- and read back by all
 // four waves.  Two buffers: chunk i + 1 is fetched into registers while chunk i
 // is computed, and written after it; one barrier per chunk.
-template <int NR, int MT>
-__global__ void __launch_bounds__(256) latent_attn_mfma_lds_kernel(LatArgs a) {
+template <int NR, int MT, int OCC>
+__global__ void __launch_bounds__(256, OCC) latent_attn_mfma_lds_kernel(LatArgs a) {
   constexpr int R = NR * 32, ND = R / 16, NF = 2 * NR + ND, NFW = NF / 4;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   bf16x8* frag = reinterpret_cast<bf16x8*>(lds_raw);          // [2][NF][64]
   __shared__ int kend_s[4];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, r = lane & 15, h = lane >> 4;
+  // ... and the LAST items of the range first: they see the most keys, so the short ones fill the tail
   const int per = gridDim.x >> 3;
-  const int blk = (gridDim.x & 7) == 0 ? (blockIdx.x & 7) * per + (blockIdx.x >> 3) : blockIdx.x;
+  const int blk = (gridDim.x & 7) == 0 ? (blockIdx.x & 7) * per + (per - 1 - (blockIdx.x >> 3))
+                                       : gridDim.x - 1 - blockIdx.x;
   const int item0 = blk * 4;
   if (item0 >= a.n_items) return;                              // whole workgroup
   const int item = item0 + wv;
@@ -522,16 +524,10 @@ static int launch_lat(const LatArgs& a, int split, int mt2, int n_head_chunks, h
   }
   if (a.n_items % 4) return (int)hipErrorInvalidValue;   // prompt items come in fours per segment
   constexpr size_t lds = 2 * (size_t)(4 * NR) * 64 * 16;  // two buffers of 2 NR + R / 16 fragments of 1 KiB
-  if constexpr (NR <= 8) {
-    if (mt2) {
-      auto k = latent_attn_mfma_lds_kernel<NR, 2>;
-      if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
-        return (int)hipGetLastError();
-      hipLaunchKernelGGL(k, grid, dim3(256), lds, s, a);
-      return (int)hipGetLastError();
-    }
-  }
-  auto k = latent_attn_mfma_lds_kernel<NR, 1>;
+  // tiles per wave and waves per SIMD by register need: two tiles while two waves still fit a SIMD
+  // (R <= 128), one tile and two waves at R = 192 / 256, one and one above
+  constexpr int MT = NR <= 4 ? 2 : 1, OCC = NR <= 8 ? 2 : 1;
+  auto k = latent_attn_mfma_lds_kernel<NR, MT, OCC>;
   if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
     return (int)hipGetLastError();
   hipLaunchKernelGGL(k, grid, dim3(256), lds, s, a);
@@ -540,10 +536,11 @@ static int launch_lat(const LatArgs& a, int split, int mt2, int n_head_chunks, h
 
 }  // namespace k8s
 
-// 1 when the MFMA kernels take latent rank R (tiles per wave for prompt portions: 2 up to R = 256).
+// 0: the MFMA kernels do not take latent rank R; else the tiles per wave for prompt portions (2 up to R = 128).
 K8S_API int k8s_latent_attn_mfma_ok(int R) {
   switch (R) {
-    case 32: case 64: case 96: case 128: case 192: case 256: case 384: case 512: return R <= 256 ? 2 : 1;
+    case 32: case 64: case 96: case 128: return 2;
+    case 192: case 256: case 384: case 512: return 1;
     default: return 0;
   }
 }
