@@ -72,11 +72,38 @@ __global__ void __launch_bounds__(256) router_kernel(const TA* __restrict__ h, c
   const int t = blockIdx.x * 4 + wv;
   if (t >= T) return;
   float* sc = sm + wv * E;
-  for (int e = 0; e < E; ++e) {
-    float a = 0.f;
-    for (int c = lane; c < W; c += 64) a = fmaf(ldx(h, (size_t)t * W + c), ldx(wr, (size_t)e * W + c), a);
-    a = wave_sum(a);
-    if (lane == 0) sc[e] = a;
+  if ((W & 7) == 0) {
+    // 8 columns per lane and step, 16 experts at a time: the hidden row is read once per group
+    for (int e0 = 0; e0 < E; e0 += 16) {
+      float acc[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) acc[j] = 0.f;
+      for (int c = lane * 8; c < W; c += 512) {
+        float hv[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) hv[i] = ldx(h, (size_t)t * W + c + i);
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+          if (e0 + j < E) {
+            const size_t wo = (size_t)(e0 + j) * W + c;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[j] = fmaf(hv[i], ldx(wr, wo + i), acc[j]);
+          }
+      }
+#pragma unroll
+      for (int j = 0; j < 16; ++j)
+        if (e0 + j < E) {
+          const float a = wave_sum(acc[j]);
+          if (lane == 0) sc[e0 + j] = a;
+        }
+    }
+  } else {
+    for (int e = 0; e < E; ++e) {
+      float a = 0.f;
+      for (int c = lane; c < W; c += 64) a = fmaf(ldx(h, (size_t)t * W + c), ldx(wr, (size_t)e * W + c), a);
+      a = wave_sum(a);
+      if (lane == 0) sc[e] = a;
+    }
   }
   __builtin_amdgcn_wave_barrier();
   if (lane == 0) {

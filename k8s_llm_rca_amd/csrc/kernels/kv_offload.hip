@@ -67,12 +67,11 @@ K8S_API int k8s_kv_stage(void* k, void* v, void* stage, long slab_bytes, int L, 
   return (int)hipGetLastError();
 }
 
-// The tier's host buffer is an ordinary allocation page-locked here (torch's
-// pinned allocator rounds every request up to a power of two: 96 GB would pin 128).
-K8S_API int k8s_host_register(void* p, long bytes) {
-  return (int)hipHostRegister(p, (size_t)bytes, hipHostRegisterDefault);
-}
-K8S_API int k8s_host_unregister(void* p) { return (int)hipHostUnregister(p); }
+// The tier's host buffer is allocated page-locked here, at its exact size (torch's
+// pinned allocator rounds every request up to a power of two: 96 GB would pin 128;
+// page-locking an existing allocation afterwards is refused on some hosts).
+K8S_API int k8s_host_alloc(void** p, long bytes) { return (int)hipHostMalloc(p, (size_t)bytes, hipHostMallocDefault); }
+K8S_API int k8s_host_free(void* p) { return (int)hipHostFree(p); }
 
 // stage <-> host slots by the DMA engines (registered host memory, so the copy
 // is asynchronous on `s`)

@@ -63,9 +63,9 @@ def _runs(ids: List[int]) -> List[Tuple[int, int, int]]:
     return out
 
 
-def _unregister(host: torch.Tensor) -> None:
+def _host_free(addr: int) -> None:
     from ..ops._lib import lib
-    lib().k8s_host_unregister(host.data_ptr())
+    lib().k8s_host_free(addr)
 
 
 class KVHostTier:
@@ -81,18 +81,23 @@ class KVHostTier:
         self.block_bytes = self.block_elems * k.element_size()
         self.host_blocks = host_blocks
         t0 = time.perf_counter()
-        self.host = torch.empty(host_blocks, self.block_elems, dtype=k.dtype)
         self._registered = False
-        if self.cuda:  # page-locked in place (k8s_host_register): DMA-able, no power-of-two rounding
+        if self.cuda:  # page-locked at its exact size (k8s_host_alloc): DMA-able, no power-of-two rounding
+            import ctypes
             from ..ops._lib import check, lib
-            print(f"[kv_host] locking {self.host.numel() * self.host.element_size() / 1e9:.1f} GB of host memory",
-                  file=sys.stderr, flush=True)
-            check(lib().k8s_host_register(self.host.data_ptr(), self.host.numel() * self.host.element_size()),
-                  "k8s_host_register")
+            nbytes = host_blocks * self.block_bytes
+            print(f"[kv_host] allocating {nbytes / 1e9:.1f} GB of page-locked host memory", file=sys.stderr,
+                  flush=True)
+            addr = ctypes.c_void_p()
+            check(lib().k8s_host_alloc(ctypes.byref(addr), nbytes), "k8s_host_alloc")
+            buf = (ctypes.c_char * nbytes).from_address(addr.value)
+            self.host = torch.frombuffer(buf, dtype=torch.uint8).view(k.dtype).view(host_blocks, self.block_elems)
             self._registered = True
-            # unlocked when the tier is collected (never at interpreter exit: the OS reclaims it)
-            self._fin = weakref.finalize(self, _unregister, self.host)
+            # freed when the tier is collected (never at interpreter exit: the OS reclaims it)
+            self._fin = weakref.finalize(self, _host_free, addr.value)
             self._fin.atexit = False
+        else:
+            self.host = torch.empty(host_blocks, self.block_elems, dtype=k.dtype)
         self.t_pin = time.perf_counter() - t0
         self._free: List[int] = list(range(host_blocks - 1, -1, -1))
         self.chunk = max(1, min(MAX_IDS, staging_bytes // self.block_bytes))
