@@ -208,7 +208,8 @@ __global__ void __launch_bounds__(256) mingru_chunk_apply_kernel(const float* __
 }
 
 // x <- unit_rms(alpha x + y) * (1 + w), in place on the fp32 residual.
-// y == nullptr: x <- unit_rms(x) * (1 + w) into `out` (the model's last norm).
+// y == nullptr: the sublayer is absent (x <- unit_rms(alpha x) * (1 + w)); with `out` the normed
+// row goes there instead of x (the model's last norm, alpha = 1: x is left as it is).
 template <typename TY, typename TW, typename TO>
 __global__ void __launch_bounds__(256) postnorm_kernel(float* __restrict__ x, const TY* __restrict__ y,
                                                        const TW* __restrict__ w, TO* __restrict__ out, int W,
@@ -218,8 +219,8 @@ __global__ void __launch_bounds__(256) postnorm_kernel(float* __restrict__ x, co
   float ss = 0.f;
   for (int c = threadIdx.x; c < W; c += 256) {
     float v = x[o + c];
-    if (y) {
-      v = fmaf(alpha, v, ldf(y, o + c));
+    if (y || alpha != 1.f) {
+      v = y ? fmaf(alpha, v, ldf(y, o + c)) : alpha * v;
       x[o + c] = v;
     }
     ss = fmaf(v, v, ss);

@@ -249,9 +249,11 @@ class ZasapelModel:
         t = random_tensors(self.cfg, seed, self.device)
         self.load_tensors(t.__getitem__)
 
-    def load_tensors(self, get) -> None:
+    def load_tensors(self, get, has=None) -> None:
         """Build the fused device layout from checkpoint tensors (``get(name)`` -> tensor, names of the
-        safetensors file: ``embed``, ``l<i>.norm1``, ``l<i>.mix.dq`` ...)."""
+        safetensors file: ``embed``, ``l<i>.norm1``, ``l<i>.mix.dq`` ...; ``has(name)`` tells what the
+        file holds).  A layer without a feed-forward whose checkpoint still carries a second norm keeps
+        that norm as an empty second sublayer."""
         cfg, dev, dt = self.cfg, self.device, self.dtype
 
         def put(*names, dtype=dt):
@@ -285,6 +287,8 @@ class ZasapelModel:
                     L["uk16"] = put(p + "mix.uk").view(H, D, KR).contiguous()
                 L["uv_t"] = put(p + "mix.uv").view(H, V, KR).transpose(1, 2).contiguous()
                 L["wo"] = put(p + "mix.o")
+            if ff is None and has is not None and has(p + "norm2"):
+                L["norm2"] = put(p + "norm2")
             if ff is not None:
                 L["norm2"], L["canon2"] = put(p + "norm2"), put(p + "canon2")
                 if ff.kind == "dense":
@@ -369,6 +373,8 @@ class ZasapelModel:
                 h = S.canon_conv(x, L["canon2"], states[f"conv{c2}"], seg, self.dtype)
                 y = self._dense(li, h) if ff.kind == "dense" else self._moe(li, h)
                 S.postnorm_(x, y, L["norm2"], cfg.postln_alpha, cfg.rms_eps)
+            elif "norm2" in L:
+                S.postnorm_(x, None, L["norm2"], cfg.postln_alpha, cfg.rms_eps)
             if layers_out is not None:
                 layers_out.append(x.clone())
         sel = x.index_select(0, inp.logits_idx)   # wanted rows in the caller's order (any permutation)
@@ -436,7 +442,7 @@ def load_checkpoint(path: str, device, dtype, pc=None) -> ZasapelModel:
         cfg = ZasapelConfig.from_json(json.load(f), name=os.path.basename(os.path.normpath(path)) or "zasapel")
     model = ZasapelModel(cfg, device, dtype, pc, init=False)
     with safe_open(os.path.join(path, "model.safetensors"), framework="pt", device="cpu") as h:
-        model.load_tensors(h.get_tensor)
+        model.load_tensors(h.get_tensor, set(h.keys()).__contains__)
     return model
 
 

@@ -176,15 +176,16 @@ def mingru_scan(zug: torch.Tensor, bz: torch.Tensor, bu: torch.Tensor, state: to
     return y
 
 
-def postnorm_(x: torch.Tensor, y: torch.Tensor, w: torch.Tensor, alpha: float, eps: float) -> torch.Tensor:
-    """In place on the fp32 residual: ``x <- unit_rms(alpha x + y) * (1 + w)``."""
+def postnorm_(x: torch.Tensor, y: Optional[torch.Tensor], w: torch.Tensor, alpha: float, eps: float) -> torch.Tensor:
+    """In place on the fp32 residual: ``x <- unit_rms(alpha x + y) * (1 + w)`` (``y`` None: no sublayer output)."""
     T, W = x.shape
     if use_hip(x):
-        assert x.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous() and y.shape == x.shape
-        check(lib().k8s_postnorm(ptr(x), ptr(y), _dt(y.dtype), ptr(w), _dt(w.dtype), None, T, W, float(alpha),
-                                 float(eps), stream_ptr(x)), "postnorm")
+        assert x.dtype == torch.float32 and x.is_contiguous()
+        assert y is None or (y.is_contiguous() and y.shape == x.shape)
+        check(lib().k8s_postnorm(ptr(x), ptr(y), 1 if y is None else _dt(y.dtype), ptr(w), _dt(w.dtype), None, T, W,
+                                 float(alpha), float(eps), stream_ptr(x)), "postnorm")
         return x
-    v = alpha * x + y.float()
+    v = alpha * x + (y.float() if y is not None else 0.0)
     x.copy_(v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * (1.0 + w.float()))
     return x
 

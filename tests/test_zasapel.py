@@ -566,6 +566,9 @@ ODD = {
     "two-latent-groups": config([(attn(kv_rank=16), None), (attn(kv_rank=32, heads=5), dense(24)),
                                  (attn(kv_rank=16, kv_from=0, heads=1), None),
                                  (attn(kv_rank=32, kv_from=1, heads=2, vdim=5), moe())], width=40, vocab=50, taps=6),
+    "unaligned": config([(attn(heads=3, dim=12, vdim=20, q_rank=36, kv_rank=40), dense(100)), (gru(60), moe(6, 2, 36, 1.0)),
+                         (attn(heads=7, dim=6, vdim=10, q_rank=18, kv_rank=40, kv_from=0), moe(3, 2, 20, 3.0))],
+                        width=100, vocab=333, taps=3),
     "top-equals-experts": config([(gru(32), moe(experts=3, top=3, ff=130, limit=0.25))], width=136, vocab=30),
 }
 
@@ -629,6 +632,34 @@ def test_thread_continues_and_restarts_when_history_diverges():
     for _ in range(3):
         seq.append(int(O.forward(d, W, seq)[-1, :eng.vocab].argmax()))
     assert out[3][:3] == seq[len(p3):]
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_second_norm_without_feed_forward(backend):
+    """A checkpoint that carries ``norm2`` for a layer without a feed-forward: the norm still applies."""
+    d = config([(attn(), None), (gru(24), None)], width=32, vocab=64)
+    W = weights(d, 24)
+    W["l0.norm2"] = (torch.randn(32, generator=torch.Generator().manual_seed(1)) * 0.2).to(torch.bfloat16).float()
+    t = toks(14, 64, 25)
+    lo = []
+    O.forward(d, W, t[:0] + t, layers_out=lo)
+    # by hand: layer 0 with the extra norm, then layer 1 and the head from the oracle's pieces
+    Wd = {k: v.double() for k, v in W.items()}
+    x = Wd["embed"][torch.tensor(t)] + O.sin_positions(len(t), 32, torch.float64)
+    h = x + O.causal_conv(x, Wd["l0.canon1"])
+    c = O.latent_of(h, Wd, "l0.mix.", 1e-5)
+    x = O.norm_zero_centered(2.5 * x + O.latent_attention(h, c, Wd, "l0.mix.", d["layers"][0]["mixer"], 1e-5), Wd["l0.norm1"], 1e-5)
+    x = O.norm_zero_centered(2.5 * x, Wd["l0.norm2"], 1e-5)
+    h = x + O.causal_conv(x, Wd["l1.canon1"])
+    x = O.norm_zero_centered(2.5 * x + O.mingru(h, Wd, "l1.mix."), Wd["l1.norm1"], 1e-5)
+    want = (O.norm_zero_centered(x, Wd["final.norm"], 1e-5) @ Wd["head"].T).float()
+    dev, dt = backend
+    model = ZasapelModel(ZasapelConfig.from_json(d, "test"), dev, dt, init=False)
+    model.load_tensors(W.__getitem__, W.__contains__)
+    eng = LLMEngine(EngineConfig(model="test", device=dev, dtype=dt, num_blocks=4, block_size=32, state_slots=2,
+                                 use_graphs=False), model=model)
+    got = feed_all(eng, eng.new_sequence(), t, (9,))
+    assert rel_err(got, want) < tol(dt)
 
 
 def test_config_round_trip_and_registry(tmp_path):
