@@ -124,7 +124,7 @@ class EngineConfig:
     model_overrides: dict = field(default_factory=dict)
     # stateful models: how many sequences can hold recurrent state at once
     # (a sequence without cached tokens needs none)
-    state_slots: int = 64
+    state_slots: int = 256
 
 
 class Request:

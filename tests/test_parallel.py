@@ -126,7 +126,11 @@ def _run_engine(rank, world, port, out_path, temperature=0.0, grammar=False, nam
         outs["_msgs"] = eng._chan.sent if eng._chan is not None else 0
         torch.save(outs, out_path)
     if world > 1:
-        dist.destroy_process_group()
+        # every rank is a spawned child: once all are done, leave without tearing the gloo group and
+        # the interpreter down (a peer closing its sockets while this rank's gloo threads still run
+        # has ended children with SIGABRT at exit, after the results were written)
+        dist.barrier()
+        os._exit(0)
 
 
 @pytest.mark.parametrize("world,name", [(2, "tiny-llama"), (4, "tiny-llama"), (8, "tiny-llama"),
