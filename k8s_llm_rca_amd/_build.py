@@ -105,7 +105,9 @@ def build_hip(force: bool = False, jobs: int = 8) -> str:
     objdir = os.path.join(PKG, "csrc", "build")
     os.makedirs(objdir, exist_ok=True)
     flags = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-munsafe-fp-atomics",
-             "-ffp-contract=fast", "-I", os.path.join(CSRC, "kernels")]
+             "-ffp-contract=fast", "-I", os.path.join(CSRC, "kernels"),
+             # no packed fp32 arithmetic (v_pk_add / mul / fma_f32): scalar forms only
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
     procs = []
     objs = []
     for s in srcs:
