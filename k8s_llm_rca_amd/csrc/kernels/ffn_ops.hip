@@ -62,16 +62,19 @@ __global__ void __launch_bounds__(256) glu_clamp_kernel(const TA* __restrict__ g
 
 // Router: one wave per token.  logits = Wr h in fp32; scores = sigmoid(logits)
 // (mode 0) or softmax (mode 1); the K largest (ties: lowest index), optionally
-// renormalised to sum 1.
+// renormalised to sum 1 (divided by their sum + renorm_eps).  With `bias` [E] the
+// choice is made on score + bias while the weights stay the plain scores.
 template <typename TA, typename TW>
 __global__ void __launch_bounds__(256) router_kernel(const TA* __restrict__ h, const TW* __restrict__ wr, int T, int W,
                                                      int E, int K, int mode, int renorm, float* __restrict__ w_out,
-                                                     int* __restrict__ id_out) {
+                                                     int* __restrict__ id_out, const float* __restrict__ bias,
+                                                     float renorm_eps) {
   extern __shared__ float sm[];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int t = blockIdx.x * 4 + wv;
   if (t >= T) return;
-  float* sc = sm + wv * E;
+  float* sc = sm + wv * 2 * E;
+  float* ch = sc + E;   // choice scores
   if ((W & 7) == 0) {
     // 8 columns per lane and step, 16 experts at a time: the hidden row is read once per group
     for (int e0 = 0; e0 < E; e0 += 16) {
@@ -115,22 +118,23 @@ __global__ void __launch_bounds__(256) router_kernel(const TA* __restrict__ h, c
       for (int e = 0; e < E; ++e) s += (sc[e] = expf(sc[e] - m));
       for (int e = 0; e < E; ++e) sc[e] /= s;
     }
+    for (int e = 0; e < E; ++e) ch[e] = bias ? sc[e] + bias[e] : sc[e];
     float tot = 0.f;
     for (int k = 0; k < K; ++k) {
       int bi = 0;
       float bv = -INFINITY;
       for (int e = 0; e < E; ++e)
-        if (sc[e] > bv) {
-          bv = sc[e];
+        if (ch[e] > bv) {
+          bv = ch[e];
           bi = e;
         }
-      w_out[t * K + k] = bv;
+      w_out[t * K + k] = sc[bi];
       id_out[t * K + k] = bi;
-      tot += bv;
-      sc[bi] = -INFINITY;
+      tot += sc[bi];
+      ch[bi] = -INFINITY;
     }
     if (renorm)
-      for (int k = 0; k < K; ++k) w_out[t * K + k] /= tot;
+      for (int k = 0; k < K; ++k) w_out[t * K + k] /= (tot + renorm_eps);
   }
 }
 
@@ -250,11 +254,12 @@ K8S_API int k8s_glu_clamp(const void* gu, void* out, int rows, int F, float alph
 }
 
 K8S_API int k8s_router(const void* h, const void* wr, int T, int W, int E, int K, int mode, int renorm, float* w_out,
-                       int* id_out, int dt, hipStream_t s) {
+                       int* id_out, int dt, hipStream_t s, const float* bias, float renorm_eps) {
   if (T <= 0) return 0;
   if (K > E || E > 2048) return (int)hipErrorInvalidValue;
-  K8S_DT(dt, hipLaunchKernelGGL((router_kernel<TA, TW>), dim3((T + 3) / 4), dim3(256), 4 * E * sizeof(float), s,
-                                 (const TA*)h, (const TW*)wr, T, W, E, K, mode, renorm, w_out, id_out));
+  K8S_DT(dt, hipLaunchKernelGGL((router_kernel<TA, TW>), dim3((T + 3) / 4), dim3(256), 8 * E * sizeof(float), s,
+                                 (const TA*)h, (const TW*)wr, T, W, E, K, mode, renorm, w_out, id_out, bias,
+                                 renorm_eps));
   return (int)hipGetLastError();
 }
 

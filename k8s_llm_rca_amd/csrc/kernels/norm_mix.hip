@@ -1,0 +1,214 @@
+// Layer norms around an fp32 residual stream, and the weighted sum over depth.
+//
+// One workgroup per row; the row is held in LDS (W floats) between the passes:
+// mean, then the mean of the squared deviations (the variance exactly as it is
+// defined, no E[x^2] - mean^2 cancellation), then the output.  Residual rows,
+// sublayer outputs and all small parameters (weights, biases, coefficients) are
+// fp32; TA is the activation type written for the next GEMM (bf16 as uint16_t,
+// or float).
+#include "common.h"
+
+namespace k8s {
+
+template <typename T>
+__device__ __forceinline__ float ldn(const T* p, size_t i);
+template <>
+__device__ __forceinline__ float ldn<float>(const float* p, size_t i) { return p[i]; }
+template <>
+__device__ __forceinline__ float ldn<uint16_t>(const uint16_t* p, size_t i) { return bf2f(p[i]); }
+template <typename T>
+__device__ __forceinline__ void stn(T* p, size_t i, float v);
+template <>
+__device__ __forceinline__ void stn<float>(float* p, size_t i, float v) { p[i] = v; }
+template <>
+__device__ __forceinline__ void stn<uint16_t>(uint16_t* p, size_t i, float v) { p[i] = f2bf(v); }
+
+// mean and 1 / sqrt(var + eps) of the LDS row (all threads get both)
+__device__ __forceinline__ void row_stats(const float* row, int W, float eps, float* red, float& mean, float& rstd) {
+  float s = 0.f;
+  for (int c = threadIdx.x; c < W; c += 256) s += row[c];
+  mean = block_sum(s, red) / (float)W;
+  float q = 0.f;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    const float d = row[c] - mean;
+    q = fmaf(d, d, q);
+  }
+  rstd = 1.f / sqrtf(block_sum(q, red) / (float)W + eps);
+}
+
+// 1 / sqrt(mean(v^2) + eps) of a global fp32 row
+__device__ __forceinline__ float row_rrms(const float* v, int W, float eps, float* red) {
+  float q = 0.f;
+  for (int c = threadIdx.x; c < W; c += 256) q = fmaf(v[c], v[c], q);
+  return 1.f / sqrtf(block_sum(q, red) / (float)W + eps);
+}
+
+template <typename TA>
+__global__ void __launch_bounds__(256) layernorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                        const float* __restrict__ b, TA* __restrict__ out, int W,
+                                                        float eps) {
+  extern __shared__ float row[];
+  __shared__ float red[16];
+  const size_t o = (size_t)blockIdx.x * W;
+  for (int c = threadIdx.x; c < W; c += 256) row[c] = x[o + c];
+  __syncthreads();
+  float mean, rstd;
+  row_stats(row, W, eps, red, mean, rstd);
+  for (int c = threadIdx.x; c < W; c += 256) stn(out, o + c, (row[c] - mean) * rstd * w[c] + b[c]);
+}
+
+// x_out = LN(embed[id]; w, b); optionally h = LN(x_out; nw, nb).
+template <typename TE, typename TA>
+__global__ void __launch_bounds__(256) embed_ln_kernel(const int* __restrict__ ids, const TE* __restrict__ embed,
+                                                       const float* __restrict__ w, const float* __restrict__ b,
+                                                       float* __restrict__ x_out, const float* __restrict__ nw,
+                                                       const float* __restrict__ nb, TA* __restrict__ h, int W,
+                                                       float eps) {
+  extern __shared__ float row[];
+  __shared__ float red[16];
+  const size_t o = (size_t)blockIdx.x * W, e0 = (size_t)ids[blockIdx.x] * W;
+  for (int c = threadIdx.x; c < W; c += 256) row[c] = ldn(embed, e0 + c);
+  __syncthreads();
+  float mean, rstd;
+  row_stats(row, W, eps, red, mean, rstd);
+  __syncthreads();
+  for (int c = threadIdx.x; c < W; c += 256) {
+    const float v = (row[c] - mean) * rstd * w[c] + b[c];
+    row[c] = v;
+    x_out[o + c] = v;
+  }
+  if (nw == nullptr) return;
+  __syncthreads();
+  row_stats(row, W, eps, red, mean, rstd);
+  for (int c = threadIdx.x; c < W; c += 256) stn(h, o + c, (row[c] - mean) * rstd * nw[c] + nb[c]);
+}
+
+// dst = src + LN(u; w, b); u = y (mode 0), (unit_rms(y) wl + unit_rms(y2) wr) / 2 (mode 1), y + y2 (mode 2).
+// Optionally h = LN(dst; nw, nb).
+template <typename TA>
+__global__ void __launch_bounds__(256) ln_residual_kernel(const float* src, const float* __restrict__ y,
+                                                          const float* __restrict__ y2, int mode,
+                                                          const float* __restrict__ wl, const float* __restrict__ wr,
+                                                          const float* __restrict__ w, const float* __restrict__ b,
+                                                          float* dst, const float* __restrict__ nw,
+                                                          const float* __restrict__ nb, TA* __restrict__ h, int W,
+                                                          float eps) {
+  extern __shared__ float row[];
+  __shared__ float red[16];
+  const size_t o = (size_t)blockIdx.x * W;
+  if (mode == 1) {
+    const float ra = row_rrms(y + o, W, eps, red), rb = row_rrms(y2 + o, W, eps, red);
+    for (int c = threadIdx.x; c < W; c += 256) row[c] = 0.5f * (y[o + c] * ra * wl[c] + y2[o + c] * rb * wr[c]);
+  } else if (mode == 2) {
+    for (int c = threadIdx.x; c < W; c += 256) row[c] = y[o + c] + y2[o + c];
+  } else {
+    for (int c = threadIdx.x; c < W; c += 256) row[c] = y[o + c];
+  }
+  __syncthreads();
+  float mean, rstd;
+  row_stats(row, W, eps, red, mean, rstd);
+  __syncthreads();
+  for (int c = threadIdx.x; c < W; c += 256) {
+    const float v = src[o + c] + ((row[c] - mean) * rstd * w[c] + b[c]);
+    row[c] = v;
+    dst[o + c] = v;
+  }
+  if (nw == nullptr) return;
+  __syncthreads();
+  row_stats(row, W, eps, red, mean, rstd);
+  for (int c = threadIdx.x; c < W; c += 256) stn(h, o + c, (row[c] - mean) * rstd * nw[c] + nb[c]);
+}
+
+// a = sum_{j < n} coef[j] * stack[j][row]; h = LN(a; w, b).  stack: [n][T][W]; rows: optional gather.
+template <typename TA>
+__global__ void __launch_bounds__(256) depth_mix_ln_kernel(const float* __restrict__ stack, size_t plane, int n,
+                                                           const float* __restrict__ coef,
+                                                           const int* __restrict__ rows, float* __restrict__ a_out,
+                                                           const float* __restrict__ w, const float* __restrict__ b,
+                                                           TA* __restrict__ h, int W, float eps) {
+  extern __shared__ float row[];
+  __shared__ float red[16];
+  const size_t r = rows ? (size_t)rows[blockIdx.x] : (size_t)blockIdx.x;
+  const size_t o = (size_t)blockIdx.x * W;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    float a = 0.f;
+    for (int j = 0; j < n; ++j) a = fmaf(coef[j], stack[(size_t)j * plane + r * W + c], a);
+    row[c] = a;
+    a_out[o + c] = a;
+  }
+  __syncthreads();
+  float mean, rstd;
+  row_stats(row, W, eps, red, mean, rstd);
+  for (int c = threadIdx.x; c < W; c += 256) stn(h, o + c, (row[c] - mean) * rstd * w[c] + b[c]);
+}
+
+__global__ void __launch_bounds__(256) softcap_kernel(float* __restrict__ z, size_t n, float scale, float cap) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const float v = z[i] * scale;
+  z[i] = cap > 0.f ? cap * tanhf(v / cap) : v;
+}
+
+}  // namespace k8s
+
+using namespace k8s;
+
+#define K8S_ODT(dt, ...)   \
+  if ((dt) == 0) {          \
+    using TA = uint16_t;    \
+    __VA_ARGS__;            \
+  } else {                  \
+    using TA = float;       \
+    __VA_ARGS__;            \
+  }
+
+static inline bool row_fits(int W) { return W > 0 && (size_t)W * sizeof(float) <= 64 * 1024; }
+
+K8S_API int k8s_layernorm(const float* x, const float* w, const float* b, void* out, int T, int W, float eps, int dt,
+                          hipStream_t s) {
+  if (T <= 0) return 0;
+  if (!row_fits(W)) return (int)hipErrorInvalidValue;
+  K8S_ODT(dt, hipLaunchKernelGGL((layernorm_kernel<TA>), dim3(T), dim3(256), W * sizeof(float), s, x, w, b, (TA*)out,
+                                 W, eps));
+  return (int)hipGetLastError();
+}
+
+K8S_API int k8s_embed_ln(const int* ids, const void* embed, int edt, const float* w, const float* b, float* x_out,
+                         const float* nw, const float* nb, void* h, int dt, int T, int W, float eps, hipStream_t s) {
+  if (T <= 0) return 0;
+  if (!row_fits(W)) return (int)hipErrorInvalidValue;
+  if (edt == 0) {
+    K8S_ODT(dt, hipLaunchKernelGGL((embed_ln_kernel<uint16_t, TA>), dim3(T), dim3(256), W * sizeof(float), s, ids,
+                                   (const uint16_t*)embed, w, b, x_out, nw, nb, (TA*)h, W, eps));
+  } else {
+    K8S_ODT(dt, hipLaunchKernelGGL((embed_ln_kernel<float, TA>), dim3(T), dim3(256), W * sizeof(float), s, ids,
+                                   (const float*)embed, w, b, x_out, nw, nb, (TA*)h, W, eps));
+  }
+  return (int)hipGetLastError();
+}
+
+K8S_API int k8s_ln_residual(const float* src, const float* y, const float* y2, int mode, const float* wl,
+                            const float* wr, const float* w, const float* b, float* dst, const float* nw,
+                            const float* nb, void* h, int dt, int T, int W, float eps, hipStream_t s) {
+  if (T <= 0) return 0;
+  if (!row_fits(W) || (mode != 0 && y2 == nullptr) || (mode == 1 && (!wl || !wr))) return (int)hipErrorInvalidValue;
+  K8S_ODT(dt, hipLaunchKernelGGL((ln_residual_kernel<TA>), dim3(T), dim3(256), W * sizeof(float), s, src, y, y2, mode,
+                                 wl, wr, w, b, dst, nw, nb, (TA*)h, W, eps));
+  return (int)hipGetLastError();
+}
+
+K8S_API int k8s_depth_mix_ln(const float* stack, int T, int n, const float* coef, const int* rows, int R,
+                             float* a_out, const float* w, const float* b, void* h, int dt, int W, float eps,
+                             hipStream_t s) {
+  if (R <= 0) return 0;
+  if (!row_fits(W) || n < 1) return (int)hipErrorInvalidValue;
+  K8S_ODT(dt, hipLaunchKernelGGL((depth_mix_ln_kernel<TA>), dim3(R), dim3(256), W * sizeof(float), s, stack,
+                                 (size_t)T * W, n, coef, rows, a_out, w, b, (TA*)h, W, eps));
+  return (int)hipGetLastError();
+}
+
+K8S_API int k8s_softcap(float* z, long n, float scale, float cap, hipStream_t s) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(softcap_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, z, (size_t)n, scale, cap);
+  return (int)hipGetLastError();
+}

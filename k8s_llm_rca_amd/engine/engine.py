@@ -38,6 +38,7 @@ import torch
 
 from ..knobs import KNOBS
 from ..models.config import ModelConfig, get_config
+from ..models.registry import OWN_CONFIG as _OWN_CONFIG
 from ..ops import attention as A
 from ..parallel.groups import ParallelContext, single
 from .graph_runner import GraphRunnerMixin
@@ -75,7 +76,7 @@ class LLMEngine(SchedulerMixin, StepExecMixin, GraphRunnerMixin, SamplerMixin):
             from ..models.registry import load_model
             model = load_model(cfg.weights, self.device, cfg.dtype, self.pc)  # the class config.json names
             self.mc = model.cfg
-        elif model is not None and getattr(getattr(model, "cfg", None), "arch", None) == "zasapel":
+        elif model is not None and getattr(getattr(model, "cfg", None), "arch", None) in _OWN_CONFIG:
             self.mc = model.cfg  # built by the caller from its own configuration
         else:
             from ..models.registry import get_any_config

@@ -162,6 +162,28 @@ class LatentKVPool(KVPool):
         return (self.c, self.ct)
 
 
+class WindowKVPool(KVPool):
+    """The same page allocator over token-major key / value pages of layers whose attention reads
+    whole rows per key: ``k[i]`` ``[num_blocks, block_size, widths[i][0]]`` and ``v[i]``
+    ``[num_blocks, block_size, widths[i][1]]`` per attention layer (its key / value heads side by side;
+    layers may differ in size).  A page index means the same token range in every tensor."""
+
+    def __init__(self, widths: List[Tuple[int, int]], num_blocks: int, block_size: int, device,
+                 dtype=torch.bfloat16):
+        self.widths = [(int(a), int(b)) for a, b in widths]
+        super().__init__(len(self.widths), 1, 0, num_blocks, block_size, device, dtype)
+
+    def _alloc_storage(self, device, dtype) -> None:
+        self.k = self.v = None
+        nb, BS = self.num_blocks, self.block_size
+        # zero-filled: a stale page never holds a NaN
+        self.kc = [torch.zeros(nb, BS, a, dtype=dtype, device=device) for a, _ in self.widths]
+        self.vc = [torch.zeros(nb, BS, b, dtype=dtype, device=device) for _, b in self.widths]
+
+    def tensors(self) -> tuple:
+        return (self.kc, self.vc)
+
+
 class StatePool:
     """Fixed-size per-sequence state beside the pages: ``slots`` slots of every
     tensor a model declares (``spec``: name -> shape behind the slot dimension),

@@ -241,8 +241,7 @@ class StepExecMixin:
         return header, flat
 
     def _exec_segments(self, header: np.ndarray, flat_host: np.ndarray, flat_dev: torch.Tensor):
-        from ..models.zasapel import SegStepInputs
-        from ..ops.seq_ops import SegMeta
+        from ..ops.seq_ops import SegMeta, SegStepInputs
         _, _, T, n_dec_rows, n, maxb, ns = [int(v) for v in header[:7]]
         o = 0
 

@@ -162,14 +162,7 @@ PRESETS: Dict[str, ZasapelConfig] = {
 }
 
 
-@dataclass
-class SegStepInputs:
-    """One step in the segment layout (:class:`..ops.seq_ops.SegMeta`)."""
-    input_ids: torch.Tensor        # [T] int32
-    positions: torch.Tensor        # [T] int32
-    slots: torch.Tensor            # [T] int32 cache slot (page * BS + offset) of every row
-    seg: S.SegMeta
-    logits_idx: torch.Tensor       # [n] int64 rows whose logits are needed
+SegStepInputs = S.SegStepInputs   # the segment-layout step (its home is ops/seq_ops.py)
 
 
 class ZasapelModel:

@@ -93,10 +93,20 @@ _SIGS = {
     "k8s_latent_attn_rows": [P, P, P, I, P, P, P, P, I, P, I, I, I, I, I, F, I, P],
     "k8s_polynorm": [P, P, P, I, I, F, I, P],
     "k8s_glu_clamp": [P, P, I, I, F, F, F, I, P],
-    "k8s_router": [P, P, I, I, I, I, I, I, P, P, I, P],
+    "k8s_router": [P, P, I, I, I, I, I, I, P, P, I, P, P, F],
     "k8s_moe_gather": [P, P, P, P, I, I, I, I, P],
     "k8s_moe_combine_f32": [P, P, P, P, I, I, I, I, P],
     "k8s_grouped_any": [P, P, P, P, I, I, I, I, I, P],
+    "k8s_layernorm": [P, P, P, P, I, I, F, I, P],
+    "k8s_embed_ln": [P, P, I, P, P, P, P, P, P, I, I, I, F, P],
+    "k8s_ln_residual": [P, P, P, I, P, P, P, P, P, P, P, P, I, I, I, F, P],
+    "k8s_depth_mix_ln": [P, I, I, P, P, I, P, P, P, P, I, I, F, P],
+    "k8s_softcap": [P, ctypes.c_long, F, F, P],
+    "k8s_short_conv": [P, I, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
+    "k8s_selective_scan": [P, I, P, P, P, I, I, P, P, P, I, P, P, P, P, P, I, I, I, I, P],
+    "k8s_retention": [P, I, P, P, P, P, P, P, P, I, I, I, I, I, F, F, I, P],
+    "k8s_window_kv_write": [P, I, I, I, I, P, P, P, I, I, P],
+    "k8s_window_attn_rows": [P, I, P, P, P, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
     "k8s_walks": [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P, P, P, P],
 }
 # entry points whose C return type is not int

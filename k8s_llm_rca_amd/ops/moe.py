@@ -158,10 +158,13 @@ def _dt(t: torch.dtype) -> int:
 
 
 def route_direct(h: torch.Tensor, w_router: torch.Tensor, k: int, scoring: str = "sigmoid",
-                 renorm: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+                 renorm: bool = False, choice_bias: Optional[torch.Tensor] = None,
+                 renorm_eps: float = 0.0) -> Tuple[torch.Tensor, torch.Tensor]:
     """Router straight from the hidden rows: fp32 logits ``h @ w_router.T``, scores by ``scoring``
-    ("sigmoid" or "softmax"), the ``k`` largest (ties: lowest index), renormalised to sum 1 only
-    with ``renorm``.  Returns (weights fp32 [T, k], ids int32 [T, k])."""
+    ("sigmoid" or "softmax"), the ``k`` largest (ties: lowest index), renormalised only with
+    ``renorm`` (divided by their sum + ``renorm_eps``).  With ``choice_bias`` (fp32 [E]) the experts
+    are chosen by score + bias while the weights are the plain scores.
+    Returns (weights fp32 [T, k], ids int32 [T, k])."""
     T, W = h.shape
     E = w_router.shape[0]
     if use_hip(h):
@@ -169,15 +172,17 @@ def route_direct(h: torch.Tensor, w_router: torch.Tensor, k: int, scoring: str =
         w = torch.empty(T, k, dtype=torch.float32, device=h.device)
         ids = torch.empty(T, k, dtype=torch.int32, device=h.device)
         check(lib().k8s_router(ptr(h), ptr(w_router), T, W, E, k, 0 if scoring == "sigmoid" else 1, int(renorm),
-                               ptr(w), ptr(ids), _dt(h.dtype), stream_ptr(h)), "router")
+                               ptr(w), ptr(ids), _dt(h.dtype), stream_ptr(h), ptr(choice_bias), float(renorm_eps)),
+              "router")
         return w, ids
     z = h.float() @ w_router.float().t()
     s = torch.sigmoid(z) if scoring == "sigmoid" else torch.softmax(z, -1)
     # stable descending sort: equal scores keep the lower expert first
-    order = torch.sort(s, dim=-1, descending=True, stable=True).indices[:, :k]
+    c = s if choice_bias is None else s + choice_bias.float()
+    order = torch.sort(c, dim=-1, descending=True, stable=True).indices[:, :k]
     w = torch.gather(s, 1, order)
     if renorm:
-        w = w / w.sum(-1, keepdim=True)
+        w = w / (w.sum(-1, keepdim=True) + renorm_eps)
     return w, order.int()
 
 

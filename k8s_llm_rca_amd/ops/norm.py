@@ -95,3 +95,127 @@ def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float, out_dtype) -> torc
 
     out.copy_((a * unit(z) + b * unit(z * z) + c * unit(z * z * z) + e).to(out_dtype))
     return out
+
+
+# ------------------------------------------------------------------ layer norms around an fp32 residual
+# (csrc/kernels/norm_mix.hip).  The residual stream, the sublayer outputs and every small
+# parameter (norm weights and biases, depth coefficients) are fp32; ``out_dtype`` is the
+# activation type that the next GEMM reads.
+def _odt(t: torch.dtype) -> int:
+    if t == torch.bfloat16:
+        return 0
+    if t == torch.float32:
+        return 1
+    raise TypeError(f"activations must be bfloat16 or float32, not {t}")
+
+
+def _ln(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float) -> torch.Tensor:
+    mu = x.mean(-1, keepdim=True)
+    d = x - mu
+    return d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps) * w + b
+
+
+def layernorm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
+    """``(x - mean) / sqrt(var + eps) * w + b`` of fp32 rows (two passes: the variance is the mean of the
+    squared deviations)."""
+    T, W = x.shape
+    out = torch.empty(T, W, dtype=out_dtype, device=x.device)
+    if use_hip(x):
+        assert x.dtype == torch.float32 and x.is_contiguous() and w.dtype == b.dtype == torch.float32
+        check(lib().k8s_layernorm(ptr(x), ptr(w), ptr(b), ptr(out), T, W, float(eps), _odt(out_dtype),
+                                  stream_ptr(x)), "layernorm")
+        return out
+    out.copy_(_ln(x, w, b, eps).to(out_dtype))
+    return out
+
+
+def embed_layernorm(ids: torch.Tensor, embed: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float,
+                    x_out: torch.Tensor, nw: Optional[torch.Tensor] = None, nb: Optional[torch.Tensor] = None,
+                    out_dtype=None) -> Optional[torch.Tensor]:
+    """``x_out = LN(embed[ids]; w, b)`` (fp32); with ``nw, nb`` also returns ``LN(x_out; nw, nb)`` as
+    activations (the first layer's input norm, same pass)."""
+    T, W = ids.shape[0], embed.shape[1]
+    h = torch.empty(T, W, dtype=out_dtype, device=embed.device) if nw is not None else None
+    if use_hip(embed):
+        assert x_out.dtype == torch.float32 and x_out.is_contiguous() and x_out.shape == (T, W)
+        assert embed.is_contiguous() and ids.dtype == torch.int32
+        check(lib().k8s_embed_ln(ptr(ids), ptr(embed), _odt(embed.dtype), ptr(w), ptr(b), ptr(x_out), ptr(nw),
+                                 ptr(nb), ptr(h), _odt(out_dtype) if h is not None else 1, T, W, float(eps),
+                                 stream_ptr(embed)), "embed_ln")
+        return h
+    x_out.copy_(_ln(embed[ids.long()].float(), w, b, eps))
+    if h is not None:
+        h.copy_(_ln(x_out, nw, nb, eps).to(out_dtype))
+    return h
+
+
+def ln_residual(src: torch.Tensor, y: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float,
+                dst: torch.Tensor, y2: Optional[torch.Tensor] = None, merge: Optional[str] = None,
+                mw: Optional[tuple] = None, nw: Optional[torch.Tensor] = None, nb: Optional[torch.Tensor] = None,
+                out_dtype=None) -> Optional[torch.Tensor]:
+    """``dst = src + LN(u; w, b)`` on fp32 rows (``dst`` may be ``src``), where ``u`` is the sublayer
+    output ``y``, or two outputs joined: ``merge="sum"``: ``y + y2``; ``merge="rms"``:
+    ``(unit_rms(y) mw[0] + unit_rms(y2) mw[1]) / 2``.  With ``nw, nb`` also returns ``LN(dst; nw, nb)`` as
+    activations (the next sublayer's input norm, same pass)."""
+    T, W = src.shape
+    h = torch.empty(T, W, dtype=out_dtype, device=src.device) if nw is not None else None
+    mode = {None: 0, "rms": 1, "sum": 2}[merge if y2 is not None else None]
+    if use_hip(src):
+        for t in (src, y, dst) + ((y2,) if y2 is not None else ()):
+            assert t.dtype == torch.float32 and t.is_contiguous() and t.shape == (T, W)
+        wl, wr = mw if mode == 1 else (None, None)
+        check(lib().k8s_ln_residual(ptr(src), ptr(y), ptr(y2), mode, ptr(wl), ptr(wr), ptr(w), ptr(b), ptr(dst),
+                                    ptr(nw), ptr(nb), ptr(h), _odt(out_dtype) if h is not None else 1, T, W,
+                                    float(eps), stream_ptr(src)), "ln_residual")
+        return h
+    if mode == 1:
+        def unit(v):
+            return v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+        u = 0.5 * (unit(y) * mw[0] + unit(y2) * mw[1])
+    elif mode == 2:
+        u = y + y2
+    else:
+        u = y
+    dst.copy_(src + _ln(u, w, b, eps))
+    if h is not None:
+        h.copy_(_ln(dst, nw, nb, eps).to(out_dtype))
+    return h
+
+
+def depth_mix_ln(stack: torch.Tensor, n: int, coef: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float,
+                 out_dtype, a_out: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None):
+    """Weighted sum over depth: ``a = sum_{j < n} coef[j] * stack[j]`` (``stack`` [>= n, T, W] fp32 holds the
+    embedding output and every layer's result) and its layer norm ``LN(a; w, b)`` as activations, one
+    pass.  ``rows`` (int64 / int32 indices): only those rows, in that order.  Returns (a, h)."""
+    _, T, W = stack.shape
+    R = T if rows is None else rows.shape[0]
+    if a_out is None:
+        a_out = torch.empty(R, W, dtype=torch.float32, device=stack.device)
+    h = torch.empty(R, W, dtype=out_dtype, device=stack.device)
+    if use_hip(stack):
+        assert stack.dtype == torch.float32 and stack.is_contiguous() and coef.dtype == torch.float32
+        assert a_out.is_contiguous() and a_out.shape == (R, W) and n <= coef.shape[0] and n <= stack.shape[0]
+        ri = None if rows is None else rows.to(torch.int32)
+        check(lib().k8s_depth_mix_ln(ptr(stack), T, n, ptr(coef), ptr(ri), R, ptr(a_out), ptr(w), ptr(b), ptr(h),
+                                     _odt(out_dtype), W, float(eps), stream_ptr(stack)), "depth_mix_ln")
+        return a_out, h
+    a = torch.zeros(T, W)
+    for j in range(n):
+        a += coef[j] * stack[j]
+    if rows is not None:
+        a = a[rows.long()]
+    a_out.copy_(a)
+    h.copy_(_ln(a_out, w, b, eps).to(out_dtype))
+    return a_out, h
+
+
+def softcap_(logits: torch.Tensor, scale: float, cap: float) -> torch.Tensor:
+    """In place on fp32 logits: ``cap * tanh(scale * z / cap)`` (``cap`` <= 0: only the scale)."""
+    if use_hip(logits):
+        assert logits.dtype == torch.float32 and logits.is_contiguous()
+        check(lib().k8s_softcap(ptr(logits), logits.numel(), float(scale), float(cap), stream_ptr(logits)), "softcap")
+        return logits
+    logits.mul_(scale)
+    if cap > 0:
+        logits.copy_(cap * torch.tanh(logits / cap))
+    return logits

@@ -11,6 +11,7 @@ the activation / weight type (bf16 or fp32).
 """
 from __future__ import annotations
 
+import math
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Tuple
 
@@ -304,4 +305,184 @@ def latent_attention(qa: torch.Tensor, cache: torch.Tensor, gate: torch.Tensor, 
         sc = sc.masked_fill(~vis[:, None, :], float("-inf"))
         o = torch.einsum("thj,jr->thr", torch.softmax(sc, -1), c)
         out[a:b] = (o * torch.sigmoid(gate[a:b, :H])[:, :, None]).to(out_dtype)
+    return out
+
+
+# ------------------------------------------------------------------ recurrent mixers and window attention
+# (csrc/kernels/mixer_ops.hip, window_attn.hip).  Small parameters (convolution taps, biases, decays,
+# A, D, the distance bias and the head-mixing matrix) are fp32 tensors.
+@dataclass
+class SegStepInputs:
+    """One step in the segment layout (:class:`SegMeta`)."""
+    input_ids: torch.Tensor        # [T] int32
+    positions: torch.Tensor        # [T] int32
+    slots: torch.Tensor            # [T] int32 cache slot (page * BS + offset) of every row
+    seg: SegMeta
+    logits_idx: torch.Tensor       # [n] int64 rows whose logits are needed
+
+
+def short_conv(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor], tail: torch.Tensor, seg: SegMeta,
+               act: bool = True) -> torch.Tensor:
+    """Causal per-channel convolution with bias and SiLU: ``out_t = act(b + sum_j w[:, j] x_(t - taps + 1 + j))``
+    over each sequence (the last column of ``w`` [C, taps] is the current token's; zeros before the
+    start).  ``x`` [T, C] may be a column slice of a wider matrix.  ``tail`` [slots, taps - 1, C] fp32
+    holds every sequence's last inputs and is advanced by this step's rows."""
+    T, C = x.shape
+    taps = w.shape[1]
+    out = torch.empty(T, C, dtype=x.dtype, device=x.device)
+    if use_hip(x):
+        assert x.stride(1) == 1 and w.dtype == torch.float32 and w.is_contiguous() and tail.is_contiguous()
+        assert tail.shape[1:] == (taps - 1, C) and 1 <= taps <= 16 and (b is None or b.dtype == torch.float32)
+        d = _dt(x.dtype)
+        check(lib().k8s_short_conv(ptr(x), x.stride(0), d, ptr(w), ptr(b), ptr(tail), ptr(seg.row_seg),
+                                   ptr(seg.seg_row0), ptr(seg.seg_pos0), ptr(seg.seg_slot), ptr(out), T, seg.n_seg, C,
+                                   taps, int(act), d, stream_ptr(x)), "short_conv")
+        return out
+    nt = taps - 1
+    xf = x.float()
+    for s in range(seg.n_seg):
+        a, e, p0, sl = seg.row0_host[s], seg.row0_host[s + 1], seg.pos0_host[s], seg.slot_host[s]
+        prev = tail[sl] if p0 > 0 else torch.zeros(nt, C)
+        ext = torch.cat([prev, xf[a:e]])
+        acc = torch.zeros(e - a, C) if b is None else b.expand(e - a, C).clone()
+        for j in range(taps):
+            acc += w[:, j] * ext[j:j + (e - a)]
+        out[a:e] = (torch.nn.functional.silu(acc) if act else acc).to(x.dtype)
+        if nt:
+            tail[sl] = ext[-nt:]
+    return out
+
+
+def selective_scan(xc: torch.Tensor, dtp: torch.Tensor, dt_bias: torch.Tensor, dbc: torch.Tensor, R: int,
+                   A: torch.Tensor, D: torch.Tensor, z: torch.Tensor, state: torch.Tensor, seg: SegMeta) -> torch.Tensor:
+    """Diagonal selective state-space recurrence per channel c and state n, fp32:
+    ``dt = softplus(dtp + dt_bias)``; ``S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n``;
+    ``y_c = (sum_n S[c, n] C_n + D_c x_c) * silu(z_c)``.  ``dbc`` [T, >= R + 2N] fp32 holds B at column R
+    and C at column R + N; ``dtp`` [T, C] fp32; ``xc`` [T, C] and ``z`` (a column slice) activations.
+    ``state`` [slots, C, N] fp32 is read (past position 0) and advanced."""
+    T, C = xc.shape
+    N = A.shape[1]
+    y = torch.empty(T, C, dtype=xc.dtype, device=xc.device)
+    if use_hip(xc):
+        assert xc.is_contiguous() and dtp.dtype == torch.float32 and dtp.is_contiguous() and dtp.shape == (T, C)
+        assert dbc.dtype == torch.float32 and dbc.stride(1) == 1 and dbc.shape[1] >= R + 2 * N
+        assert z.stride(1) == 1 and z.dtype == xc.dtype and state.is_contiguous() and state.shape[1:] == (C, N)
+        assert A.dtype == D.dtype == dt_bias.dtype == torch.float32 and A.is_contiguous()
+        check(lib().k8s_selective_scan(ptr(xc), _dt(xc.dtype), ptr(dtp), ptr(dt_bias), ptr(dbc), dbc.stride(0), R,
+                                       ptr(A), ptr(D), ptr(z), z.stride(0), ptr(state), ptr(seg.seg_row0),
+                                       ptr(seg.seg_pos0), ptr(seg.seg_slot), ptr(y), seg.n_seg, C, N, T,
+                                       stream_ptr(xc)), "selective_scan")
+        return y
+    dt = torch.nn.functional.softplus(dtp + dt_bias)
+    xf, zf = xc.float(), z.float()
+    Bm, Cm = dbc[:, R:R + N], dbc[:, R + N:R + 2 * N]
+    for s in range(seg.n_seg):
+        a, e, p0, sl = seg.row0_host[s], seg.row0_host[s + 1], seg.pos0_host[s], seg.slot_host[s]
+        S = state[sl].clone() if p0 > 0 else torch.zeros(C, N)
+        for r in range(a, e):
+            S = torch.exp(dt[r][:, None] * A) * S + (dt[r] * xf[r])[:, None] * Bm[r][None, :]
+            y[r] = ((S @ Cm[r] + D * xf[r]) * torch.nn.functional.silu(zf[r])).to(xc.dtype)
+        state[sl] = S
+    return y
+
+
+def retention(qkvg: torch.Tensor, H: int, D: int, V: int, decay: torch.Tensor, rot_dims: int, rot_base: float,
+              state: torch.Tensor, seg: SegMeta, positions: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
+    """Retention per head, fp32: rows of ``qkvg`` [T, 2HD + 2HV] fp32 = (q | k | v | g).  q and k are
+    rotated on their first ``rot_dims`` entries (entry i paired with i + rot_dims / 2, angle
+    ``pos * rot_base^(-2i / rot_dims)``), k is scaled by ``D^(-1/2)``; ``S <- decay_h S + k v^T``;
+    ``o = S^T q``; the result is ``o / rms(o) * silu(g)`` [T, H * V].  ``state`` [slots, H, D, V] fp32."""
+    T = qkvg.shape[0]
+    out = torch.empty(T, H * V, dtype=out_dtype, device=qkvg.device)
+    if use_hip(qkvg):
+        assert qkvg.dtype == torch.float32 and qkvg.stride(1) == 1 and qkvg.shape[1] == 2 * H * (D + V)
+        assert state.is_contiguous() and state.shape[1:] == (H, D, V) and decay.dtype == torch.float32
+        check(lib().k8s_retention(ptr(qkvg), qkvg.stride(0), ptr(positions), ptr(decay), ptr(state), ptr(seg.seg_row0),
+                                  ptr(seg.seg_pos0), ptr(seg.seg_slot), ptr(out), seg.n_seg, H, D, V, rot_dims,
+                                  float(rot_base), float(eps), _dt(out_dtype), stream_ptr(qkvg)), "retention")
+        return out
+    half = rot_dims // 2
+    f = torch.exp(-(2.0 * torch.arange(half, dtype=torch.float64) / max(rot_dims, 1)) * math.log(rot_base))
+    ang = positions.double()[:, None] * f[None]
+    co, si = ang.cos().float()[:, None, :], ang.sin().float()[:, None, :]
+
+    def rot(x):
+        u, v = x[..., :half], x[..., half:rot_dims]
+        return torch.cat([u * co - v * si, v * co + u * si, x[..., rot_dims:]], -1)
+
+    q = rot(qkvg[:, :H * D].view(T, H, D))
+    k = rot(qkvg[:, H * D:2 * H * D].view(T, H, D)) * D ** -0.5
+    v = qkvg[:, 2 * H * D:2 * H * D + H * V].view(T, H, V)
+    g = qkvg[:, 2 * H * D + H * V:].view(T, H, V)
+    for s in range(seg.n_seg):
+        a, e, p0, sl = seg.row0_host[s], seg.row0_host[s + 1], seg.pos0_host[s], seg.slot_host[s]
+        S = state[sl].clone() if p0 > 0 else torch.zeros(H, D, V)
+        for r in range(a, e):
+            S = decay[:, None, None] * S + k[r][:, :, None] * v[r][:, None, :]
+            o = torch.einsum("hdv,hd->hv", S, q[r])
+            o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * torch.nn.functional.silu(g[r])
+            out[r] = o.reshape(-1).to(out_dtype)
+        state[sl] = S
+    return out
+
+
+def window_kv_write(qkv: torch.Tensor, k_off: int, kc: torch.Tensor, vc: torch.Tensor, slots: torch.Tensor) -> None:
+    """The key and value columns of the joint projection's rows (k at ``k_off``, v behind it) go to the
+    pages ``kc`` [pages, BS, G D] / ``vc`` [pages, BS, G V] at ``slots`` (page * BS + offset)."""
+    T = qkv.shape[0]
+    nk, nv = kc.shape[-1], vc.shape[-1]
+    if use_hip(qkv):
+        assert qkv.stride(1) == 1 and kc.is_contiguous() and vc.is_contiguous() and kc.dtype == vc.dtype == qkv.dtype
+        assert qkv.shape[1] >= k_off + nk + nv
+        check(lib().k8s_window_kv_write(ptr(qkv), qkv.stride(0), k_off, nk, nv, ptr(slots), ptr(kc), ptr(vc), T,
+                                        _dt(qkv.dtype), stream_ptr(qkv)), "window_kv_write")
+        return
+    ok = slots >= 0
+    sl = slots[ok].long()
+    kc.view(-1, nk)[sl] = qkv[ok, k_off:k_off + nk]
+    vc.view(-1, nv)[sl] = qkv[ok, k_off + nk:k_off + nk + nv]
+
+
+def window_attention(qkv: torch.Tensor, H: int, G: int, D: int, V: int, kc: torch.Tensor, vc: torch.Tensor,
+                     r1: torch.Tensor, r2: torch.Tensor, talk: torch.Tensor, window: int, scale: float,
+                     seg: SegMeta) -> torch.Tensor:
+    """Sliding-window attention of the rows' queries (the first H D columns of ``qkv``) over the paged
+    keys and values, which already hold this step's rows: position i sees j with ``0 <= i - j < window``;
+    ``s = scale q.k - r1[h] ln(1 + r2[h] (i - j))``; ``p_j = exp(s_j) / (1 + sum exp(s))`` (a sink of score 0
+    without a value); the heads' weights are mixed, ``w_h = sum_g talk[h, g] p_g``, and head h applies
+    its mixed weights to the values of key / value head ``h // (H // G)``.  Returns [T, H V]."""
+    T = qkv.shape[0]
+    BS = kc.shape[1]
+    out = torch.empty(T, H * V, dtype=qkv.dtype, device=qkv.device)
+    if use_hip(qkv):
+        assert qkv.stride(1) == 1 and kc.is_contiguous() and vc.is_contiguous() and kc.dtype == vc.dtype == qkv.dtype
+        assert kc.shape[-1] == G * D and vc.shape[-1] == G * V and seg.block_tables.is_contiguous()
+        assert r1.dtype == r2.dtype == talk.dtype == torch.float32 and talk.is_contiguous() and H % G == 0
+        check(lib().k8s_window_attn_rows(ptr(qkv), qkv.stride(0), ptr(kc), ptr(vc), ptr(seg.block_tables),
+                                         seg.block_tables.shape[1], ptr(seg.row_seg), ptr(seg.seg_row0),
+                                         ptr(seg.seg_pos0), ptr(r1), ptr(r2), ptr(talk), ptr(out), T, H, G, D, V, BS,
+                                         int(window), float(scale), _dt(qkv.dtype), stream_ptr(qkv)),
+              "window_attn_rows")
+        return out
+    kf, vf = kc.view(-1, G, D), vc.view(-1, G, V)
+    rep = H // G
+    for s in range(seg.n_seg):
+        a, e, p0 = seg.row0_host[s], seg.row0_host[s + 1], seg.pos0_host[s]
+        n, n_ctx = e - a, p0 + e - a
+        lo = max(0, p0 - window + 1)
+        kp = torch.arange(lo, n_ctx)
+        rows = seg.block_tables[s].long()[kp // BS] * BS + kp % BS
+        k = kf[rows].float().repeat_interleave(rep, 1)             # [ctx, H, D]
+        v = vf[rows].float().repeat_interleave(rep, 1)             # [ctx, H, V]
+        q = qkv[a:e, :H * D].float().view(n, H, D)
+        dist = (p0 + torch.arange(n))[:, None] - kp[None, :]       # [n, ctx]
+        sc = torch.einsum("thd,jhd->thj", q, k) * scale
+        sc = sc - r1[None, :, None] * torch.log1p(r2[None, :, None] * dist.clamp_min(0).float()[:, None, :])
+        vis = (dist >= 0) & (dist < window)
+        sc = sc.masked_fill(~vis[:, None, :], float("-inf"))
+        m = sc.amax(-1, keepdim=True).clamp_min(0.0)
+        ex = torch.exp(sc - m)
+        p = ex / (torch.exp(-m) + ex.sum(-1, keepdim=True))
+        pm = torch.einsum("hg,tgj->thj", talk, p)
+        out[a:e] = torch.einsum("thj,jhv->thv", pm, v).reshape(n, H * V).to(qkv.dtype)
     return out
