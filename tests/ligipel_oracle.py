@@ -24,15 +24,11 @@ def rms(x, eps):
     return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
 
 
-def window_attention(h, w, p, m, dt):
-    """Sliding window, log-distance bias, softmax with a zero-score sink, heads' weights mixed."""
-    T = h.shape[0]
-    H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    win, scale = m["mask"]["size"], m["scale"]
-    q = (h @ w[p + "q"].to(dt).T).view(T, H, D)
-    k = (h @ w[p + "k"].to(dt).T).view(T, G, D)
-    v = (h @ w[p + "v"].to(dt).T).view(T, G, V)
-    r1, r2, talk = w[p + "r1"].to(dt), w[p + "r2"].to(dt), w[p + "talk"].to(dt)
+def window_attention_core(q, k, v, r1, r2, talk, win, scale):
+    """q [T, H, D], k [T, G, D], v [T, G, V] of one sequence -> [T, H, V]."""
+    T, H, _ = q.shape
+    G, V = k.shape[1], v.shape[2]
+    dt = q.dtype
     P = torch.zeros(H, T, T, dtype=dt)
     for hh in range(H):
         g = hh // (H // G)
@@ -46,29 +42,52 @@ def window_attention(h, w, p, m, dt):
     out = torch.zeros(T, H, V, dtype=dt)
     for hh in range(H):
         out[:, hh] = Pm[hh] @ v[:, hh // (H // G)]
+    return out
+
+
+def window_attention(h, w, p, m, dt):
+    """Sliding window, log-distance bias, softmax with a zero-score sink, heads' weights mixed."""
+    T = h.shape[0]
+    H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    q = (h @ w[p + "q"].to(dt).T).view(T, H, D)
+    k = (h @ w[p + "k"].to(dt).T).view(T, G, D)
+    v = (h @ w[p + "v"].to(dt).T).view(T, G, V)
+    out = window_attention_core(q, k, v, w[p + "r1"].to(dt), w[p + "r2"].to(dt), w[p + "talk"].to(dt),
+                                m["mask"]["size"], m["scale"])
     return out.reshape(T, H * V) @ w[p + "o"].to(dt).T
 
 
-def mamba(h, w, p, m, dt):
-    T = h.shape[0]
-    C, N, R, taps = m["inner"], m["state"], m["dt_rank"], m["conv"]
-    xz = h @ w[p + "in"].to(dt).T
-    x, z = xz[:, :C], xz[:, C:]
-    cw, cb = w[p + "conv"].to(dt), w[p + "conv.b"].to(dt)
-    xp = torch.cat([torch.zeros(taps - 1, C, dtype=dt), x])
-    xc = torch.zeros(T, C, dtype=dt)
+def causal_conv_silu(x, cw, cb):
+    """x [T, C], cw [C, taps] (last column: the current token), cb [C]."""
+    T, C = x.shape
+    taps = cw.shape[1]
+    xp = torch.cat([torch.zeros(taps - 1, C, dtype=x.dtype), x])
+    out = torch.zeros(T, C, dtype=x.dtype)
     for t in range(T):
-        xc[t] = (xp[t:t + taps] * cw.T).sum(0) + cb
-    xc = F.silu(xc)
-    dbc = xc @ w[p + "x"].to(dt).T
-    dlt = F.softplus(dbc[:, :R] @ w[p + "dt"].to(dt).T + w[p + "dt.b"].to(dt))
-    B, Cm = dbc[:, R:R + N], dbc[:, R + N:R + 2 * N]
-    A = -torch.exp(w[p + "A_log"].to(dt))
-    S = torch.zeros(C, N, dtype=dt)
-    y = torch.zeros(T, C, dtype=dt)
+        out[t] = (xp[t:t + taps] * cw.T).sum(0) + cb
+    return F.silu(out)
+
+
+def selective_scan(xc, dlt, A, B, Cm, D):
+    """xc, dlt [T, C]; A [C, N]; B, Cm [T, N]; D [C] -> y [T, C] (before the gate)."""
+    T, C = xc.shape
+    S = torch.zeros(C, A.shape[1], dtype=xc.dtype)
+    y = torch.zeros(T, C, dtype=xc.dtype)
     for t in range(T):
         S = torch.exp(dlt[t][:, None] * A) * S + (dlt[t] * xc[t])[:, None] * B[t][None, :]
-        y[t] = S @ Cm[t] + w[p + "D"].to(dt) * xc[t]
+        y[t] = S @ Cm[t] + D * xc[t]
+    return y
+
+
+def mamba(h, w, p, m, dt):
+    C, N, R = m["inner"], m["state"], m["dt_rank"]
+    xz = h @ w[p + "in"].to(dt).T
+    x, z = xz[:, :C], xz[:, C:]
+    xc = causal_conv_silu(x, w[p + "conv"].to(dt), w[p + "conv.b"].to(dt))
+    dbc = xc @ w[p + "x"].to(dt).T
+    dlt = F.softplus(dbc[:, :R] @ w[p + "dt"].to(dt).T + w[p + "dt.b"].to(dt))
+    A = -torch.exp(w[p + "A_log"].to(dt))
+    y = selective_scan(xc, dlt, A, dbc[:, R:R + N], dbc[:, R + N:R + 2 * N], w[p + "D"].to(dt))
     return (y * F.silu(z)) @ w[p + "o"].to(dt).T
 
 
@@ -88,6 +107,18 @@ def rotate(x, pos, dims, base, dt):
     return torch.cat([u * c - v * s, v * c + u * s, x[..., dims:]], -1)
 
 
+def retention_core(q, k, v, decay):
+    """q, k [T, H, D] (rotated, k scaled), v [T, H, V] -> o [T, H, V]."""
+    T, H, D = q.shape
+    o = torch.zeros(T, H, v.shape[2], dtype=q.dtype)
+    for hh in range(H):
+        S = torch.zeros(D, v.shape[2], dtype=q.dtype)
+        for t in range(T):
+            S = decay[hh] * S + k[t, hh][:, None] * v[t, hh][None, :]
+            o[t, hh] = S.T @ q[t, hh]
+    return o
+
+
 def retention(h, w, p, m, eps, dt):
     T = h.shape[0]
     H, D, V = m["heads"], m["dim"], m["vdim"]
@@ -95,12 +126,7 @@ def retention(h, w, p, m, eps, dt):
     q = rotate((h @ w[p + "q"].to(dt).T).view(T, H, D), pos, m["rot"]["dims"], m["rot"]["base"], dt)
     k = rotate((h @ w[p + "k"].to(dt).T).view(T, H, D), pos, m["rot"]["dims"], m["rot"]["base"], dt) * D ** -0.5
     v = (h @ w[p + "v"].to(dt).T).view(T, H, V)
-    o = torch.zeros(T, H, V, dtype=dt)
-    for hh in range(H):
-        S = torch.zeros(D, V, dtype=dt)
-        for t in range(T):
-            S = m["decay"][hh] * S + k[t, hh][:, None] * v[t, hh][None, :]
-            o[t, hh] = S.T @ q[t, hh]
+    o = retention_core(q, k, v, m["decay"])
     o = rms(o, eps).reshape(T, H * V) * F.silu(h @ w[p + "g"].to(dt).T)
     return o @ w[p + "o"].to(dt).T
 
@@ -109,11 +135,15 @@ def expert(h, w, p, dt):
     return (F.silu(h @ w[p + "gate"].to(dt).T) * (h @ w[p + "up"].to(dt).T)) @ w[p + "down"].to(dt).T
 
 
+def route(h, wr, corr, top):
+    """(softmax scores [T, E], chosen experts [T, top]): chosen by score + correction."""
+    s = torch.softmax(h @ wr.T, -1)
+    return s, torch.topk(s + corr, top, dim=-1).indices
+
+
 def moe(h, w, p, f, dt):
-    E, top = f["router"]["experts"], f["router"]["top"]
-    s = torch.softmax(h @ w[p + "router"].to(dt).T, -1)
-    choice = s + w[p + "correction"].to(dt)
-    idx = torch.topk(choice, top, dim=-1).indices
+    top = f["router"]["top"]
+    s, idx = route(h, w[p + "router"].to(dt), w[p + "correction"].to(dt), top)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         sel = s[t, idx[t]]
@@ -152,6 +182,6 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens: List[int], dt=torch.f
         x = sum(d[j] * X[j] for j in range(i + 2))
         if layers_out is not None:
             layers_out.append(x.clone())
-    z = ln(x, "final.norm") @ w["head"].to(dt).T * cfg["logit_scale"]
-    cap = cfg["logit_softcap"]
-    return cap * torch.tanh(z / cap)
+    z = ln(x, "final.norm") @ w["head"].to(dt).T * cfg.get("logit_scale", 1.0)
+    cap = cfg.get("logit_softcap", 0.0)
+    return cap * torch.tanh(z / cap) if cap else z
