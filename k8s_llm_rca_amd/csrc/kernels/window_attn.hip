@@ -26,16 +26,22 @@ __device__ __forceinline__ void stw<float>(float* p, size_t i, float v) { p[i] =
 template <>
 __device__ __forceinline__ void stw<uint16_t>(uint16_t* p, size_t i, float v) { p[i] = f2bf(v); }
 
-// The k and v parts of the joint projection's rows go to their pages.
+// The k and v parts of the joint projection's rows go to their pages; vt (optional) is the
+// transposed twin of the value pages, [pages][G * V][BS]: the matrix-core kernel's PV operand.
 template <typename TA>
 __global__ void __launch_bounds__(256) window_kv_write_kernel(const TA* __restrict__ qkv, int qs, int k_off, int nk,
                                                               int nv, const int* __restrict__ slots,
-                                                              TA* __restrict__ kc, TA* __restrict__ vc) {
+                                                              TA* __restrict__ kc, TA* __restrict__ vc,
+                                                              TA* __restrict__ vt, int BS) {
   const int t = blockIdx.x, sl = slots[t];
   if (sl < 0) return;
   const TA* row = qkv + (size_t)t * qs + k_off;
   for (int c = threadIdx.x; c < nk; c += 256) kc[(size_t)sl * nk + c] = row[c];
   for (int c = threadIdx.x; c < nv; c += 256) vc[(size_t)sl * nv + c] = row[nk + c];
+  if (vt) {
+    const int page = sl / BS, off = sl - page * BS;
+    for (int c = threadIdx.x; c < nv; c += 256) vt[((size_t)page * nv + c) * BS + off] = row[nk + c];
+  }
 }
 
 constexpr int kWinTile = 64;   // keys per tile: one per lane
@@ -142,6 +148,236 @@ __global__ void __launch_bounds__(256) window_attn_rows_kernel(const TA* __restr
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Matrix-core form (bf16, v_mfma_f32_16x16x32_bf16).  A workgroup of four waves owns a tile of up
+// to 16 consecutive tokens of one segment; wave w owns the heads w HW .. w HW + HW - 1.  Keys go
+// in blocks of 32 (never across a page: BS % 32 == 0).  Swapped QK^T as in the other attention
+// kernels: a lane owns ONE query (lane & 15) and, per block, the scores of keys 8 q .. 8 q + 7 of its
+// quarter q = lane >> 4 -- for every head at the same (query, key) positions, so mixing the heads'
+// weights is element-wise across heads.
+//   pass 1: per head and query the maximum (the sink's 0 included) and the denominator, online;
+//   pass 2: scores again -> normalised weights of the wave's heads -> LDS -> every wave mixes all
+//           heads' weights for its own heads (fp32) -> bf16 PV operand in place -> O += W V.
+// The weights go through LDS double-buffered: one barrier per key block.
+struct WinArgs {
+  const uint16_t* qkv;    // [T][qs], the queries in the first H * D columns
+  int qs;
+  const uint16_t* kc;     // [pages][BS][G * D]
+  const uint16_t* vt;     // [pages][G * V][BS]
+  const int* bt;
+  int maxb;
+  const int* items;       // [n][4]: segment, first row, tokens (<= 16), position of the first token
+  int n_items;
+  const float* r1;
+  const float* r2;
+  const float* talk;
+  uint16_t* out;          // [T][H * V]
+  int H, G, BS, window;
+  float scale;
+};
+
+__device__ __forceinline__ bf16x8 wld16(const uint16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+
+template <int NDC>
+__device__ __forceinline__ void win_scores(const bf16x8 (&kf)[2][NDC], const bf16x8 (&qf)[NDC], int kb, int hq,
+                                           int posq, bool qvalid, int window, float sl2, float c1, float c2,
+                                           float (&p)[8]) {
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    f32x4 sacc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int cc = 0; cc < NDC; ++cc) sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][cc], qf[cc], sacc, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int dist = posq - (kb + 8 * hq + 4 * t + i);
+      const bool ok = qvalid && dist >= 0 && dist < window;
+      // log2 units: scale q.k log2(e) - r1 log2(1 + r2 dist)
+      p[4 * t + i] = ok ? sacc[i] * sl2 - c1 * __log2f(1.f + c2 * (float)dist) : -INFINITY;
+    }
+  }
+}
+
+template <int NDC, int NV, int HW>
+__global__ void __launch_bounds__(256) window_attn_mfma_kernel(WinArgs a) {
+  constexpr int D = NDC * 32, V = NV * 16;
+  constexpr float kLog2e = 1.4426950408889634f;
+  extern __shared__ float psm[];   // [2][H][2][64][4]: the normalised weights of one key block
+  const int lane = threadIdx.x & 63, r = lane & 15, hq = lane >> 4;
+  const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int item = blockIdx.x;
+  const int sg = a.items[item * 4], row0 = a.items[item * 4 + 1], ntok = a.items[item * 4 + 2],
+            pos0 = a.items[item * 4 + 3];
+  const int H = a.H, hpg = H / a.G, NK = a.G * D, NVt = a.G * V;
+  const int h0 = wv * HW, nh = max(0, min(HW, H - h0));
+  const int posq = pos0 + r;
+  const bool qvalid = r < ntok;
+  const int k_lo = max(0, pos0 - a.window + 1), k_hi = pos0 + ntok - 1;
+  const float sl2 = a.scale * kLog2e;
+  const int* pages = a.bt + (size_t)sg * a.maxb;
+  bf16x8 qf[HW][NDC];
+  float m2[HW], l[HW], c1[HW], c2[HW], inv_l[HW];
+#pragma unroll
+  for (int hh = 0; hh < HW; ++hh) {
+    const bool on = hh < nh && qvalid;
+    const uint16_t* qp = a.qkv + (size_t)(row0 + (on ? r : 0)) * a.qs + (size_t)(on ? h0 + hh : 0) * D;
+#pragma unroll
+    for (int cc = 0; cc < NDC; ++cc) {
+      qf[hh][cc] = wld16(qp + 32 * cc + 8 * hq);
+      if (!on)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) qf[hh][cc][j] = (__bf16)0.f;
+    }
+    m2[hh] = 0.f;   // the sink's score
+    l[hh] = 0.f;
+    c1[hh] = hh < nh ? a.r1[h0 + hh] : 0.f;
+    c2[hh] = hh < nh ? a.r2[h0 + hh] : 0.f;
+  }
+  // ---- pass 1: maximum and denominator
+  for (int kb = k_lo & ~31; kb <= k_hi; kb += 32) {
+    const int page = pages[kb / a.BS], off = kb % a.BS;
+    const uint16_t* kp = a.kc + ((size_t)page * a.BS + off) * NK;
+    bf16x8 kf[2][NDC];
+    int gprev = -1;
+#pragma unroll
+    for (int hh = 0; hh < HW; ++hh) {
+      if (hh < nh) {
+        const int g = (h0 + hh) / hpg;
+        if (g != gprev) {
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            const int key = 8 * (r >> 2) + 4 * t + (r & 3);
+#pragma unroll
+            for (int cc = 0; cc < NDC; ++cc) kf[t][cc] = wld16(kp + (size_t)key * NK + g * D + 32 * cc + 8 * hq);
+          }
+          gprev = g;
+        }
+        float p[8];
+        win_scores<NDC>(kf, qf[hh], kb, hq, posq, qvalid, a.window, sl2, c1[hh], c2[hh], p);
+        float cmax = p[0];
+#pragma unroll
+        for (int j = 1; j < 8; ++j) cmax = fmaxf(cmax, p[j]);
+        cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
+        cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
+        const float mn = fmaxf(m2[hh], cmax);
+        float ps = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ps += exp2f(p[j] - mn);
+        l[hh] = l[hh] * exp2f(m2[hh] - mn) + ps;
+        m2[hh] = mn;
+      }
+    }
+  }
+#pragma unroll
+  for (int hh = 0; hh < HW; ++hh) {
+    float lt = l[hh];
+    lt += __shfl_xor(lt, 16, 64);
+    lt += __shfl_xor(lt, 32, 64);
+    inv_l[hh] = 1.f / (lt + exp2f(-m2[hh]));     // + the sink
+  }
+  // ---- pass 2: weights, mixed over heads, times the values
+  f32x4 o[HW][NV];
+#pragma unroll
+  for (int hh = 0; hh < HW; ++hh)
+#pragma unroll
+    for (int dt = 0; dt < NV; ++dt) o[hh][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  int buf = 0;
+  for (int kb = k_lo & ~31; kb <= k_hi; kb += 32) {
+    const int page = pages[kb / a.BS], off = kb % a.BS;
+    const uint16_t* kp = a.kc + ((size_t)page * a.BS + off) * NK;
+    float* P = psm + (size_t)buf * H * 512;
+    {
+      bf16x8 kf[2][NDC];
+      int gprev = -1;
+#pragma unroll
+      for (int hh = 0; hh < HW; ++hh) {
+        if (hh < nh) {
+          const int g = (h0 + hh) / hpg;
+          if (g != gprev) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+              const int key = 8 * (r >> 2) + 4 * t + (r & 3);
+#pragma unroll
+              for (int cc = 0; cc < NDC; ++cc) kf[t][cc] = wld16(kp + (size_t)key * NK + g * D + 32 * cc + 8 * hq);
+            }
+            gprev = g;
+          }
+          float p[8];
+          win_scores<NDC>(kf, qf[hh], kb, hq, posq, qvalid, a.window, sl2, c1[hh], c2[hh], p);
+          float* Ph = P + (size_t)(h0 + hh) * 512 + lane * 4;
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            f32x4 e;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) e[i] = exp2f(p[4 * t + i] - m2[hh]) * inv_l[hh];
+            *reinterpret_cast<f32x4*>(Ph + t * 256) = e;
+          }
+        }
+      }
+    }
+    __syncthreads();
+    bf16x8 vf[NV];
+    int gprev = -1;
+#pragma unroll
+    for (int hh = 0; hh < HW; ++hh) {
+      if (hh < nh) {
+        f32x4 w0 = f32x4{0.f, 0.f, 0.f, 0.f}, w1 = w0;
+        const float* tk = a.talk + (size_t)(h0 + hh) * H;
+        for (int g2 = 0; g2 < H; ++g2) {
+          const float tv = tk[g2];
+          const f32x4 e0 = *reinterpret_cast<const f32x4*>(P + (size_t)g2 * 512 + lane * 4);
+          const f32x4 e1 = *reinterpret_cast<const f32x4*>(P + (size_t)g2 * 512 + 256 + lane * 4);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            w0[i] = fmaf(tv, e0[i], w0[i]);
+            w1[i] = fmaf(tv, e1[i], w1[i]);
+          }
+        }
+        bf16x8 pf;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          pf[i] = (__bf16)w0[i];
+          pf[4 + i] = (__bf16)w1[i];
+        }
+        const int g = (h0 + hh) / hpg;
+        if (g != gprev) {
+          const uint16_t* vp = a.vt + ((size_t)page * NVt + (size_t)g * V) * a.BS + off + 8 * hq;
+#pragma unroll
+          for (int dt = 0; dt < NV; ++dt) vf[dt] = wld16(vp + (size_t)(16 * dt + r) * a.BS);
+          gprev = g;
+        }
+#pragma unroll
+        for (int dt = 0; dt < NV; ++dt) o[hh][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf[dt], o[hh][dt], 0, 0, 0);
+      }
+    }
+    buf ^= 1;
+  }
+#pragma unroll
+  for (int hh = 0; hh < HW; ++hh) {
+    if (hh < nh) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int q = 4 * hq + i;
+        if (q < ntok) {
+          uint16_t* op = a.out + (size_t)(row0 + q) * H * V + (size_t)(h0 + hh) * V + r;
+#pragma unroll
+          for (int dt = 0; dt < NV; ++dt) op[16 * dt] = f2bf(o[hh][dt][i]);
+        }
+      }
+    }
+  }
+}
+
+template <int NDC, int NV, int HW>
+static int launch_win_mfma(const WinArgs& a, hipStream_t s) {
+  const size_t lds = (size_t)2 * a.H * 512 * sizeof(float);
+  auto k = window_attn_mfma_kernel<NDC, NV, HW>;
+  if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
+    return (int)hipGetLastError();
+  hipLaunchKernelGGL(k, dim3(a.n_items), dim3(256), lds, s, a);
+  return (int)hipGetLastError();
+}
+
 }  // namespace k8s
 
 using namespace k8s;
@@ -156,11 +392,51 @@ using namespace k8s;
   }
 
 K8S_API int k8s_window_kv_write(const void* qkv, int qs, int k_off, int nk, int nv, const int* slots, void* kc,
-                                void* vc, int T, int dt, hipStream_t s) {
+                                void* vc, int T, int dt, hipStream_t s, void* vt, int BS) {
   if (T <= 0) return 0;
+  if (vt && BS <= 0) return (int)hipErrorInvalidValue;
   K8S_WDT(dt, hipLaunchKernelGGL((window_kv_write_kernel<TA>), dim3(T), dim3(256), 0, s, (const TA*)qkv, qs, k_off, nk,
-                                 nv, slots, (TA*)kc, (TA*)vc));
+                                 nv, slots, (TA*)kc, (TA*)vc, (TA*)vt, BS));
   return (int)hipGetLastError();
+}
+
+// 1 when the matrix-core kernel takes these sizes (bf16 only)
+K8S_API int k8s_window_attn_mfma_ok(int H, int G, int D, int V) {
+  return H >= 1 && H <= 16 && G >= 1 && H % G == 0 && (D == 64 || D == 128) && (V == 64 || V == 128);
+}
+
+K8S_API int k8s_window_attn_mfma(const void* qkv, int qs, const void* kc, const void* vt, const int* block_tables,
+                                 int maxb, const int* items, int n_items, const float* r1, const float* r2,
+                                 const float* talk, void* out, int H, int G, int D, int V, int BS, int window,
+                                 float scale, hipStream_t s) {
+  if (n_items <= 0) return 0;
+  if (!k8s_window_attn_mfma_ok(H, G, D, V) || BS % 32 || window < 1 || qs % 8 || (D * G) % 8)
+    return (int)hipErrorInvalidValue;
+  WinArgs a;
+  a.qkv = (const uint16_t*)qkv;
+  a.qs = qs;
+  a.kc = (const uint16_t*)kc;
+  a.vt = (const uint16_t*)vt;
+  a.bt = block_tables;
+  a.maxb = maxb;
+  a.items = items;
+  a.n_items = n_items;
+  a.r1 = r1;
+  a.r2 = r2;
+  a.talk = talk;
+  a.out = (uint16_t*)out;
+  a.H = H;
+  a.G = G;
+  a.BS = BS;
+  a.window = window;
+  a.scale = scale;
+  const bool wide = H > 8;
+#define K8S_WIN(NDC, NV) (wide ? launch_win_mfma<NDC, NV, 4>(a, s) : launch_win_mfma<NDC, NV, 2>(a, s))
+  if (D == 64 && V == 64) return K8S_WIN(2, 4);
+  if (D == 64 && V == 128) return K8S_WIN(2, 8);
+  if (D == 128 && V == 64) return K8S_WIN(4, 4);
+  return K8S_WIN(4, 8);
+#undef K8S_WIN
 }
 
 K8S_API int k8s_window_attn_rows(const void* qkv, int qs, const void* kc, const void* vc, const int* block_tables,

@@ -166,11 +166,14 @@ class WindowKVPool(KVPool):
     """The same page allocator over token-major key / value pages of layers whose attention reads
     whole rows per key: ``k[i]`` ``[num_blocks, block_size, widths[i][0]]`` and ``v[i]``
     ``[num_blocks, block_size, widths[i][1]]`` per attention layer (its key / value heads side by side;
-    layers may differ in size).  A page index means the same token range in every tensor."""
+    layers may differ in size), plus the values' transposed twin ``vt[i]`` ``[num_blocks, widths[i][1],
+    block_size]`` for the layers in ``twins`` (the matrix-core attention kernel's PV operand: 8 consecutive
+    keys of one value column contiguous).  A page index means the same token range in every tensor."""
 
     def __init__(self, widths: List[Tuple[int, int]], num_blocks: int, block_size: int, device,
-                 dtype=torch.bfloat16):
+                 dtype=torch.bfloat16, twins: Optional[List[bool]] = None):
         self.widths = [(int(a), int(b)) for a, b in widths]
+        self.twins = list(twins) if twins is not None else [False] * len(self.widths)
         super().__init__(len(self.widths), 1, 0, num_blocks, block_size, device, dtype)
 
     def _alloc_storage(self, device, dtype) -> None:
@@ -179,9 +182,11 @@ class WindowKVPool(KVPool):
         # zero-filled: a stale page never holds a NaN
         self.kc = [torch.zeros(nb, BS, a, dtype=dtype, device=device) for a, _ in self.widths]
         self.vc = [torch.zeros(nb, BS, b, dtype=dtype, device=device) for _, b in self.widths]
+        self.vt = [torch.zeros(nb, b, BS, dtype=dtype, device=device) if tw else None
+                   for (_, b), tw in zip(self.widths, self.twins)]
 
     def tensors(self) -> tuple:
-        return (self.kc, self.vc)
+        return (self.kc, self.vc, self.vt)
 
 
 class StatePool:

@@ -231,12 +231,18 @@ class LigipelModel:
 
     # ------------------------------------------------------- what the engine allocates for this model
     def cache_bytes_per_block(self, block_size: int) -> int:
-        return max(1, sum(a + b for a, b in self.cache_widths)) * block_size * (2 if self.dtype == torch.bfloat16
-                                                                                 else 4)
+        per = sum(a + (2 * b if tw else b) for (a, b), tw in zip(self.cache_widths, self._twins()))
+        return max(1, per) * block_size * (2 if self.dtype == torch.bfloat16 else 4)
+
+    def _twins(self) -> List[bool]:
+        """Per attention layer: whether the matrix-core kernel runs it (then its values are also cached
+        transposed)."""
+        return [S.window_mfma_ok(L.left.heads, L.left.kv_heads, L.left.dim, L.left.vdim, self.dtype, self.device)
+                for L in self.cfg.layers if L.kind == "parallel"]
 
     def make_cache(self, num_blocks: int, block_size: int):
         from ..engine.kv_cache import WindowKVPool
-        return WindowKVPool(self.cache_widths, num_blocks, block_size, self.device, self.dtype)
+        return WindowKVPool(self.cache_widths, num_blocks, block_size, self.device, self.dtype, self._twins())
 
     def state_spec(self) -> Dict[str, Tuple[int, ...]]:
         """Per-slot fp32 state tensors: name -> shape behind the slot dimension."""
@@ -337,13 +343,14 @@ class LigipelModel:
         """x @ w.T with an fp32 result (fp32 accumulation either way)."""
         return linear_f32out(x, w) if self.dtype == torch.bfloat16 else linear(x, w)
 
-    def _window_attention(self, li: int, h: torch.Tensor, inp: S.SegStepInputs, kcs, vcs) -> torch.Tensor:
+    def _window_attention(self, li: int, h: torch.Tensor, inp: S.SegStepInputs, kcs, vcs, vts) -> torch.Tensor:
         L, a = self.layers[li], self.cfg.layers[li].left
-        kc, vc = kcs[self.cache_of[li]], vcs[self.cache_of[li]]
+        ci = self.cache_of[li]
+        kc, vc, vt = kcs[ci], vcs[ci], vts[ci]
         qkv = linear(h, L["w_qkv"])                                  # [T, H D + G D + G V]
-        S.window_kv_write(qkv, a.heads * a.dim, kc, vc, inp.slots)
+        S.window_kv_write(qkv, a.heads * a.dim, kc, vc, inp.slots, vt)
         o = S.window_attention(qkv, a.heads, a.kv_heads, a.dim, a.vdim, kc, vc, L["r1"], L["r2"], L["talk"],
-                               a.window, a.scale, inp.seg)
+                               a.window, a.scale, inp.seg, vt)
         return self._lin32(o, L["wo_l"])
 
     def _ssm(self, li: int, h: torch.Tensor, seg: S.SegMeta, states) -> torch.Tensor:
@@ -381,9 +388,10 @@ class LigipelModel:
         return routed, shared
 
     def forward(self, inp: S.SegStepInputs, kcs: List[torch.Tensor], vcs: List[torch.Tensor],
-                states: Dict[str, torch.Tensor], layers_out: Optional[list] = None) -> torch.Tensor:
+                vts: List[Optional[torch.Tensor]], states: Dict[str, torch.Tensor],
+                layers_out: Optional[list] = None) -> torch.Tensor:
         """Logits [len(logits_idx), vocab] fp32.  ``kcs`` / ``vcs``: the paged keys and values of every
-        attention layer; ``states``: the per-slot tensors of :meth:`state_spec`.  ``layers_out``
+        attention layer (``vts``: the values' transposed twins, or None); ``states``: the per-slot tensors of :meth:`state_spec`.  ``layers_out``
         (debugging): receives a copy of the residual after every layer (behind its sum over depth)."""
         cfg, eps, dt = self.cfg, self.cfg.norm_eps, self.dtype
         T, W, nl = inp.input_ids.shape[0], cfg.hidden, cfg.n_layers
@@ -394,7 +402,7 @@ class LigipelModel:
         for li, (spec, L) in enumerate(zip(cfg.layers, self.layers)):
             nxt = L["norm2"] if spec.mlp is not None else (None, None)
             if spec.kind == "parallel":
-                yl = self._window_attention(li, h, inp, kcs, vcs)
+                yl = self._window_attention(li, h, inp, kcs, vcs, vts)
                 yr = self._ssm(li, h, inp.seg, states)
                 h = N.ln_residual(a, yl, *L["norm1b"], eps, X[li + 1], y2=yr, merge="rms",
                                   mw=(L["out_l"], L["out_r"]), nw=nxt[0], nb=nxt[1], out_dtype=dt)

@@ -66,6 +66,20 @@ class SegMeta:
         return got
 
 
+    def tile_items(self, tokens_per_item: int) -> torch.Tensor:
+        """Every segment cut into tiles of at most ``tokens_per_item`` consecutive tokens ([n, 4] int32 on
+        the device: segment, first row, tokens, position of the first token), made once per step."""
+        key = ("tiles", tokens_per_item)
+        got = self._items.get(key)
+        if got is None:
+            it = [(s, r, min(tokens_per_item, self.row0_host[s + 1] - r), self.pos0_host[s] + r - self.row0_host[s])
+                  for s in range(self.n_seg) for r in range(self.row0_host[s], self.row0_host[s + 1], tokens_per_item)]
+            host = torch.from_numpy(np.asarray(it, dtype=np.int32).reshape(-1, 4))
+            if self.row_seg.device.type == "cuda":
+                host = host.pin_memory()
+            got = self._items[key] = host.to(self.row_seg.device, non_blocking=True)
+        return got
+
     def scan_chunks(self, rows: int) -> Optional[torch.Tensor]:
         """Chunks of at most ``rows`` rows for the time-parallel recurrence ([n, 4] int32 on the device:
         segment, first row, rows, index of the segment's first chunk); None when no segment is longer
@@ -426,31 +440,50 @@ def retention(qkvg: torch.Tensor, H: int, D: int, V: int, decay: torch.Tensor, r
     return out
 
 
-def window_kv_write(qkv: torch.Tensor, k_off: int, kc: torch.Tensor, vc: torch.Tensor, slots: torch.Tensor) -> None:
+def window_mfma_ok(H: int, G: int, D: int, V: int, dtype, device) -> bool:
+    """Whether the matrix-core window attention kernel takes these sizes (bf16 on the device only;
+    the vector-pipe kernel runs everything else)."""
+    if dtype != torch.bfloat16 or torch.device(device).type != "cuda":
+        return False
+    return bool(lib().k8s_window_attn_mfma_ok(int(H), int(G), int(D), int(V)))
+
+
+WINDOW_TILE = 16    # query tokens per work item of the matrix-core window attention kernel
+
+
+def window_kv_write(qkv: torch.Tensor, k_off: int, kc: torch.Tensor, vc: torch.Tensor, slots: torch.Tensor,
+                    vt: Optional[torch.Tensor] = None) -> None:
     """The key and value columns of the joint projection's rows (k at ``k_off``, v behind it) go to the
-    pages ``kc`` [pages, BS, G D] / ``vc`` [pages, BS, G V] at ``slots`` (page * BS + offset)."""
+    pages ``kc`` [pages, BS, G D] / ``vc`` [pages, BS, G V] at ``slots`` (page * BS + offset), the values
+    also to the transposed twin ``vt`` [pages, G V, BS] when given (the matrix-core kernel's PV operand)."""
     T = qkv.shape[0]
     nk, nv = kc.shape[-1], vc.shape[-1]
+    BS = kc.shape[1]
     if use_hip(qkv):
         assert qkv.stride(1) == 1 and kc.is_contiguous() and vc.is_contiguous() and kc.dtype == vc.dtype == qkv.dtype
         assert qkv.shape[1] >= k_off + nk + nv
+        assert vt is None or (vt.is_contiguous() and vt.dtype == qkv.dtype and vt.shape[1:] == (nv, BS))
         check(lib().k8s_window_kv_write(ptr(qkv), qkv.stride(0), k_off, nk, nv, ptr(slots), ptr(kc), ptr(vc), T,
-                                        _dt(qkv.dtype), stream_ptr(qkv)), "window_kv_write")
+                                        _dt(qkv.dtype), stream_ptr(qkv), ptr(vt), BS), "window_kv_write")
         return
     ok = slots >= 0
     sl = slots[ok].long()
     kc.view(-1, nk)[sl] = qkv[ok, k_off:k_off + nk]
     vc.view(-1, nv)[sl] = qkv[ok, k_off + nk:k_off + nk + nv]
+    if vt is not None:
+        vt[sl // BS, :, sl % BS] = qkv[ok, k_off + nk:k_off + nk + nv]
 
 
 def window_attention(qkv: torch.Tensor, H: int, G: int, D: int, V: int, kc: torch.Tensor, vc: torch.Tensor,
                      r1: torch.Tensor, r2: torch.Tensor, talk: torch.Tensor, window: int, scale: float,
-                     seg: SegMeta) -> torch.Tensor:
+                     seg: SegMeta, vt: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Sliding-window attention of the rows' queries (the first H D columns of ``qkv``) over the paged
     keys and values, which already hold this step's rows: position i sees j with ``0 <= i - j < window``;
     ``s = scale q.k - r1[h] ln(1 + r2[h] (i - j))``; ``p_j = exp(s_j) / (1 + sum exp(s))`` (a sink of score 0
     without a value); the heads' weights are mixed, ``w_h = sum_g talk[h, g] p_g``, and head h applies
-    its mixed weights to the values of key / value head ``h // (H // G)``.  Returns [T, H V]."""
+    its mixed weights to the values of key / value head ``h // (H // G)``.  Returns [T, H V].
+    With the transposed value pages ``vt`` (bf16, sizes of :func:`window_mfma_ok`) the matrix-core
+    kernel runs: tiles of ``WINDOW_TILE`` tokens, the weights rounded to bf16 for the value product."""
     T = qkv.shape[0]
     BS = kc.shape[1]
     out = torch.empty(T, H * V, dtype=qkv.dtype, device=qkv.device)
@@ -458,6 +491,14 @@ def window_attention(qkv: torch.Tensor, H: int, G: int, D: int, V: int, kc: torc
         assert qkv.stride(1) == 1 and kc.is_contiguous() and vc.is_contiguous() and kc.dtype == vc.dtype == qkv.dtype
         assert kc.shape[-1] == G * D and vc.shape[-1] == G * V and seg.block_tables.is_contiguous()
         assert r1.dtype == r2.dtype == talk.dtype == torch.float32 and talk.is_contiguous() and H % G == 0
+        if vt is not None and window_mfma_ok(H, G, D, V, qkv.dtype, qkv.device) and qkv.stride(0) % 8 == 0:
+            assert vt.is_contiguous() and vt.shape[1:] == (G * V, BS) and BS % 32 == 0
+            items = seg.tile_items(WINDOW_TILE)
+            check(lib().k8s_window_attn_mfma(ptr(qkv), qkv.stride(0), ptr(kc), ptr(vt), ptr(seg.block_tables),
+                                             seg.block_tables.shape[1], ptr(items), items.shape[0], ptr(r1), ptr(r2),
+                                             ptr(talk), ptr(out), H, G, D, V, BS, int(window), float(scale),
+                                             stream_ptr(qkv)), "window_attn_mfma")
+            return out
         check(lib().k8s_window_attn_rows(ptr(qkv), qkv.stride(0), ptr(kc), ptr(vc), ptr(seg.block_tables),
                                          seg.block_tables.shape[1], ptr(seg.row_seg), ptr(seg.seg_row0),
                                          ptr(seg.seg_pos0), ptr(r1), ptr(r2), ptr(talk), ptr(out), T, H, G, D, V, BS,
