@@ -92,7 +92,13 @@ __global__ void __launch_bounds__(256) short_conv_tail_kernel(const TA* __restri
 //   dt = softplus(dtp[r][c] + dt_bias[c]);  S[n] <- exp(dt A[c][n]) S[n] + dt x B[r][n];
 //   y = (sum_n S[n] C[r][n] + D[c] x) * silu(z[r][c]).
 // dbc rows (stride ds) hold B at column R and C at column R + N, fp32.  state [slots][C][N].
-template <int NMAX, typename TA>
+// MODE 0: a whole segment per workgroup row (blockIdx.x = segment), state read and written.
+// Long segments are cut into chunks ([n][4]: segment, first row, rows, -) that run in parallel:
+// MODE 1: a chunk from a zero state: its end state and the sum of its step sizes go to
+//         cs [chunks][C][N] / csd [chunks][C] (the chunk's decay is exp(A * sum dt));
+// (scan_carry_kernel then turns cs into every chunk's START state and advances the slot's state)
+// MODE 2: the chunk again from its start state, writing y.
+template <int NMAX, int MODE, typename TA>
 __global__ void __launch_bounds__(128) selective_scan_kernel(const TA* __restrict__ xc, const float* __restrict__ dtp,
                                                              const float* __restrict__ dt_bias,
                                                              const float* __restrict__ dbc, int ds, int R,
@@ -101,12 +107,24 @@ __global__ void __launch_bounds__(128) selective_scan_kernel(const TA* __restric
                                                              const int* __restrict__ seg_row0,
                                                              const int* __restrict__ seg_pos0,
                                                              const int* __restrict__ seg_slot, TA* __restrict__ y,
-                                                             int C, int N) {
-  const int sg = blockIdx.x, c = blockIdx.y * 128 + threadIdx.x;
+                                                             int C, int N, const int* __restrict__ chunks,
+                                                             float* __restrict__ cs, float* __restrict__ csd) {
+  const int it = blockIdx.x, c = blockIdx.y * 128 + threadIdx.x;
   if (c >= C) return;
-  const int r0 = seg_row0[sg], r1 = seg_row0[sg + 1];
-  const bool fresh = seg_pos0[sg] == 0;
-  float* st = state + ((size_t)seg_slot[sg] * C + c) * N;
+  int r0, r1;
+  bool fresh;
+  float* st;
+  if (MODE == 0) {
+    r0 = seg_row0[it];
+    r1 = seg_row0[it + 1];
+    fresh = seg_pos0[it] == 0;
+    st = state + ((size_t)seg_slot[it] * C + c) * N;
+  } else {
+    r0 = chunks[it * 4 + 1];
+    r1 = r0 + chunks[it * 4 + 2];
+    fresh = MODE == 1;
+    st = cs + ((size_t)it * C + c) * N;
+  }
   float S[NMAX], Ac[NMAX];
 #pragma unroll
   for (int n = 0; n < NMAX; ++n) {
@@ -114,6 +132,7 @@ __global__ void __launch_bounds__(128) selective_scan_kernel(const TA* __restric
     S[n] = (n < N && !fresh) ? st[n] : 0.f;
   }
   const float Dc = Dp[c], bias = dt_bias[c];
+  float sd = 0.f;
   for (int r = r0; r < r1; ++r) {
     const float dv = dtp[(size_t)r * C + c] + bias;
     const float dt = dv > 20.f ? dv : log1pf(expf(dv));
@@ -122,106 +141,163 @@ __global__ void __launch_bounds__(128) selective_scan_kernel(const TA* __restric
     const float* Bp = dbc + (size_t)r * ds + R;
     const float* Cp = Bp + N;
     float acc = 0.f;
+    sd += dt;
 #pragma unroll
     for (int n = 0; n < NMAX; ++n)
       if (n < N) {
         S[n] = fmaf(expf(dt * Ac[n]), S[n], dx * Bp[n]);
-        acc = fmaf(S[n], Cp[n], acc);
+        if (MODE != 1) acc = fmaf(S[n], Cp[n], acc);
       }
-    const float zv = ldm(z, (size_t)r * zs + c);
-    stm(y, (size_t)r * C + c, (acc + Dc * xv) * silu_f(zv));
+    if (MODE != 1) {
+      const float zv = ldm(z, (size_t)r * zs + c);
+      stm(y, (size_t)r * C + c, (acc + Dc * xv) * silu_f(zv));
+    }
+  }
+  if (MODE != 2) {
+#pragma unroll
+    for (int n = 0; n < NMAX; ++n)
+      if (n < N) st[n] = S[n];
+  }
+  if (MODE == 1) csd[(size_t)it * C + c] = sd;
+}
+
+// Between the two chunk passes, one thread per (segment, channel): walk the segment's chunks
+// (seg_chunk0[s] .. seg_chunk0[s + 1]), replace every chunk's end-from-zero state by its START state,
+// and leave the segment's final state in the slot.
+template <int NMAX>
+__global__ void __launch_bounds__(128) scan_carry_kernel(const float* __restrict__ A, float* __restrict__ state,
+                                                         const int* __restrict__ seg_pos0,
+                                                         const int* __restrict__ seg_slot,
+                                                         const int* __restrict__ seg_chunk0, float* __restrict__ cs,
+                                                         const float* __restrict__ csd, int C, int N) {
+  const int sg = blockIdx.x, c = blockIdx.y * 128 + threadIdx.x;
+  if (c >= C) return;
+  float* st = state + ((size_t)seg_slot[sg] * C + c) * N;
+  const bool fresh = seg_pos0[sg] == 0;
+  float S[NMAX], Ac[NMAX];
+#pragma unroll
+  for (int n = 0; n < NMAX; ++n) {
+    Ac[n] = n < N ? A[(size_t)c * N + n] : 0.f;
+    S[n] = (n < N && !fresh) ? st[n] : 0.f;
+  }
+  for (int k = seg_chunk0[sg]; k < seg_chunk0[sg + 1]; ++k) {
+    float* ck = cs + ((size_t)k * C + c) * N;
+    const float sd = csd[(size_t)k * C + c];
+#pragma unroll
+    for (int n = 0; n < NMAX; ++n)
+      if (n < N) {
+        const float loc = ck[n];
+        ck[n] = S[n];
+        S[n] = fmaf(expf(sd * Ac[n]), S[n], loc);
+      }
   }
 #pragma unroll
   for (int n = 0; n < NMAX; ++n)
     if (n < N) st[n] = S[n];
 }
 
-// Retention, one workgroup per (segment, head), token by token.  Rows of qkvg (fp32, stride qs):
-// q [H][D] | k [H][D] | v [H][V] | g [H][V].  q and k are rotated on their first `rot` entries
-// (entry i with i + rot / 2; angle = pos * base^(-2 i / rot), formed in double), k is scaled by
-// D^(-1/2);  S <- decay S + k v^T;  o = S^T q;  out = o / rms(o) * silu(g).
-// Thread (dg, v) of NDG x V owns S[d][v] for d = dg, dg + NDG, ...  state [slots][H][D][V].
-constexpr int kRetDpt = 64;
-template <typename TA>
-__global__ void __launch_bounds__(256) retention_kernel(const float* __restrict__ qkvg, int qs,
-                                                        const int* __restrict__ positions,
-                                                        const float* __restrict__ decay, float* __restrict__ state,
-                                                        const int* __restrict__ seg_row0,
-                                                        const int* __restrict__ seg_pos0,
-                                                        const int* __restrict__ seg_slot, TA* __restrict__ out, int H,
-                                                        int D, int V, int rot, float base, float eps) {
+// Retention in three kernels.  Rows of qkvg (fp32, stride qs): q [H][D] | k [H][D] | v [H][V] | g [H][V].
+//   1. retention_rope_kernel (one workgroup per token, in place): q and k are rotated on their first
+//      `rot` entries (entry i with i + rot / 2; angle = pos * base^(-2 i / rot), formed in double) and k is
+//      scaled by D^(-1/2);
+//   2. retention_scan_kernel, one workgroup per (segment, head, block of <= 64 value columns), tokens
+//      in batches of 16 through LDS:  S <- decay S + k v^T;  o = S^T q  (fp32, written raw).
+//      Thread (dg, v) of NDG x VBS owns S[d][v] for d = dg, dg + NDG, ...  state [slots][H][D][V];
+//   3. head_norm_gate_kernel: out = o / rms(o over the head's V) * silu(g).
+__global__ void __launch_bounds__(256) retention_rope_kernel(float* __restrict__ qkvg, int qs,
+                                                             const int* __restrict__ positions, int H, int D, int rot,
+                                                             float base) {
+  extern __shared__ float cs[];   // [half] cos | [half] sin
+  const int r = blockIdx.x, tid = threadIdx.x, half = rot >> 1;
+  float* row = qkvg + (size_t)r * qs;
+  const double lb = log((double)base), p = (double)positions[r];
+  for (int i = tid; i < half; i += 256) {
+    const double ang = p * exp(-(double)(2 * i) / (double)rot * lb);
+    cs[i] = (float)cos(ang);
+    cs[half + i] = (float)sin(ang);
+  }
+  __syncthreads();
+  const float ks = 1.f / sqrtf((float)D);
+  for (int e = tid; e < 2 * H * half; e += 256) {        // the rotated pairs of q (first H heads) and k
+    const int hd = e / half, i = e - hd * half;
+    float* x = row + (size_t)hd * D;
+    const float u = x[i], v = x[i + half], sc = hd >= H ? ks : 1.f;
+    x[i] = (u * cs[i] - v * cs[half + i]) * sc;
+    x[i + half] = (v * cs[i] + u * cs[half + i]) * sc;
+  }
+  const int rest = D - rot;
+  for (int e = tid; e < H * rest; e += 256) {            // k's entries behind the rotated ones
+    const int h = e / rest, i = e - h * rest;
+    row[(size_t)(H + h) * D + rot + i] *= ks;
+  }
+}
+
+constexpr int kRetDpt = 64;   // state rows per thread
+constexpr int kRetTb = 16;    // tokens per batch
+__global__ void __launch_bounds__(256) retention_scan_kernel(const float* __restrict__ qkvg, int qs,
+                                                             const float* __restrict__ decay, float* __restrict__ state,
+                                                             const int* __restrict__ seg_row0,
+                                                             const int* __restrict__ seg_pos0,
+                                                             const int* __restrict__ seg_slot, float* __restrict__ oraw,
+                                                             int H, int D, int V, int VBS) {
   extern __shared__ float sm[];
-  __shared__ float red[16];
-  const int sg = blockIdx.x, hh = blockIdx.y, tid = threadIdx.x;
-  const int NDG = 256 / V, half = rot >> 1;
-  float* sq = sm;                 // [D]
-  float* sk = sq + D;             // [D]
-  float* sv = sk + D;             // [V]
-  float* part = sv + V;           // [NDG][V]
-  float* cs = part + NDG * V;     // [half] cos | [half] sin
-  const int v = tid % V, dg = tid / V;
-  const bool own = dg < NDG;
+  const int sg = blockIdx.x, hh = blockIdx.y, v0 = blockIdx.z * VBS, tid = threadIdx.x;
+  const int NDG = 256 / VBS;
+  float* sq = sm;                          // [TB][D]
+  float* sk = sq + kRetTb * D;             // [TB][D]
+  float* sv = sk + kRetTb * D;             // [TB][VBS]
+  float* part = sv + kRetTb * VBS;         // [TB][NDG][VBS]
+  const int v = tid % VBS, dg = tid / VBS;
+  const bool own = dg < NDG && v0 + v < V;
   const int r0 = seg_row0[sg], r1 = seg_row0[sg + 1];
   const bool fresh = seg_pos0[sg] == 0;
-  float* st = state + ((size_t)seg_slot[sg] * H + hh) * D * V;
-  const float dec = decay[hh], ks = 1.f / sqrtf((float)D);
+  float* st = state + ((size_t)seg_slot[sg] * H + hh) * D * V + v0;
+  const float dec = decay[hh];
   float S[kRetDpt];
 #pragma unroll
   for (int i = 0; i < kRetDpt; ++i) {
     const int d = dg + i * NDG;
     S[i] = (own && d < D && !fresh) ? st[(size_t)d * V + v] : 0.f;
   }
-  const double lb = log((double)base);
-  for (int r = r0; r < r1; ++r) {
-    const float* row = qkvg + (size_t)r * qs;
+  for (int t0 = r0; t0 < r1; t0 += kRetTb) {
+    const int nb = min(kRetTb, r1 - t0);
     __syncthreads();
-    if (tid < half) {
-      const double ang = (double)positions[r] * exp(-(double)(2 * tid) / (double)rot * lb);
-      cs[tid] = (float)cos(ang);
-      cs[half + tid] = (float)sin(ang);
+    for (int e = tid; e < nb * D; e += 256) {
+      const int tb = e / D, d = e - tb * D;
+      const float* row = qkvg + (size_t)(t0 + tb) * qs;
+      sq[e] = row[hh * D + d];
+      sk[e] = row[(H + hh) * D + d];
+    }
+    for (int e = tid; e < nb * VBS; e += 256) {
+      const int tb = e / VBS, vv = e - tb * VBS;
+      sv[e] = v0 + vv < V ? qkvg[(size_t)(t0 + tb) * qs + 2 * H * D + hh * V + v0 + vv] : 0.f;
     }
     __syncthreads();
-    for (int d = tid; d < D; d += 256) {
-      const float* q = row + hh * D;
-      const float* k = row + (H + hh) * D;
-      float qv, kv;
-      if (d < half) {
-        qv = q[d] * cs[d] - q[d + half] * cs[half + d];
-        kv = k[d] * cs[d] - k[d + half] * cs[half + d];
-      } else if (d < rot) {
-        const int i = d - half;
-        qv = q[d] * cs[i] + q[i] * cs[half + i];
-        kv = k[d] * cs[i] + k[i] * cs[half + i];
-      } else {
-        qv = q[d];
-        kv = k[d];
-      }
-      sq[d] = qv;
-      sk[d] = kv * ks;
-    }
-    for (int i = tid; i < V; i += 256) sv[i] = row[2 * H * D + hh * V + i];
-    __syncthreads();
-    if (own) {
-      const float vv = sv[v];
-      float acc = 0.f;
+    if (dg < NDG) {
+      for (int tb = 0; tb < nb; ++tb) {
+        const float vv = sv[tb * VBS + v];
+        const float* kq = sk + tb * D;
+        const float* qq = sq + tb * D;
+        float acc = 0.f;
 #pragma unroll
-      for (int i = 0; i < kRetDpt; ++i) {
-        const int d = dg + i * NDG;
-        if (d < D) {
-          S[i] = fmaf(dec, S[i], sk[d] * vv);
-          acc = fmaf(S[i], sq[d], acc);
+        for (int i = 0; i < kRetDpt; ++i) {
+          const int d = dg + i * NDG;
+          if (d < D) {
+            S[i] = fmaf(dec, S[i], kq[d] * vv);
+            acc = fmaf(S[i], qq[d], acc);
+          }
         }
+        part[(tb * NDG + dg) * VBS + v] = acc;
       }
-      part[dg * V + v] = acc;
     }
     __syncthreads();
-    float o = 0.f;
-    if (tid < V)
-      for (int g = 0; g < NDG; ++g) o += part[g * V + tid];
-    const float ss = block_sum(tid < V ? o * o : 0.f, red);
-    if (tid < V) {
-      const float gv = row[2 * H * D + H * V + hh * V + tid];
-      stm(out, (size_t)r * H * V + hh * V + tid, o / sqrtf(ss / (float)V + eps) * silu_f(gv));
+    for (int e = tid; e < nb * VBS; e += 256) {
+      const int tb = e / VBS, vv = e - tb * VBS;
+      if (v0 + vv < V) {
+        float o = 0.f;
+        for (int g = 0; g < NDG; ++g) o += part[(tb * NDG + g) * VBS + vv];
+        oraw[(size_t)(t0 + tb) * H * V + hh * V + v0 + vv] = o;
+      }
     }
   }
 #pragma unroll
@@ -229,6 +305,22 @@ __global__ void __launch_bounds__(256) retention_kernel(const float* __restrict_
     const int d = dg + i * NDG;
     if (own && d < D) st[(size_t)d * V + v] = S[i];
   }
+}
+
+// out[r][h] = o / sqrt(mean(o^2 over V) + eps) * silu(g): one wave per (row, head).
+template <typename TA>
+__global__ void __launch_bounds__(256) head_norm_gate_kernel(const float* __restrict__ oraw,
+                                                             const float* __restrict__ gate, int gs,
+                                                             TA* __restrict__ out, int n_rh, int H, int V, float eps) {
+  const int rh = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (rh >= n_rh) return;
+  const int r = rh / H, h = rh - r * H;
+  const float* o = oraw + (size_t)rh * V;
+  float ss = 0.f;
+  for (int c = lane; c < V; c += 64) ss = fmaf(o[c], o[c], ss);
+  const float rn = 1.f / sqrtf(wave_sum(ss) / (float)V + eps);
+  const float* g = gate + (size_t)r * gs + (size_t)h * V;
+  for (int c = lane; c < V; c += 64) stm(out, (size_t)rh * V + c, o[c] * rn * silu_f(g[c]));
 }
 
 }  // namespace k8s
@@ -263,36 +355,56 @@ K8S_API int k8s_short_conv(const void* x, int xs, int xdt, const float* w, const
 K8S_API int k8s_selective_scan(const void* xc, int dt, const float* dtp, const float* dt_bias, const float* dbc,
                                int ds, int R, const float* A, const float* D, const void* z, int zs, float* state,
                                const int* seg_row0, const int* seg_pos0, const int* seg_slot, void* y, int n_seg,
-                               int C, int N, int T, hipStream_t s) {
+                               int C, int N, int T, hipStream_t s, const int* chunks, int n_chunks,
+                               const int* seg_chunk0, float* cs, float* csd) {
   if (T <= 0 || n_seg <= 0) return 0;
   if (N < 1 || N > 128) return (int)hipErrorInvalidValue;
-  const dim3 g(n_seg, (C + 127) / 128);
+  const int cb = (C + 127) / 128;
+#define K8S_SCAN_M(NM, MODE, items)                                                                               \
+  K8S_MDT(dt, hipLaunchKernelGGL((selective_scan_kernel<NM, MODE, TA>), dim3(items, cb), dim3(128), 0, s,          \
+                                 (const TA*)xc, dtp, dt_bias, dbc, ds, R, A, D, (const TA*)z, zs, state, seg_row0, \
+                                 seg_pos0, seg_slot, (TA*)y, C, N, chunks, cs, csd))
 #define K8S_SCAN(NM)                                                                                              \
-  K8S_MDT(dt, hipLaunchKernelGGL((selective_scan_kernel<NM, TA>), g, dim3(128), 0, s, (const TA*)xc, dtp, dt_bias, \
-                                 dbc, ds, R, A, D, (const TA*)z, zs, state, seg_row0, seg_pos0, seg_slot, (TA*)y, \
-                                 C, N))
+  if (chunks == nullptr) {                                                                                        \
+    K8S_SCAN_M(NM, 0, n_seg);                                                                                     \
+  } else {                                                                                                        \
+    K8S_SCAN_M(NM, 1, n_chunks);                                                                                  \
+    hipLaunchKernelGGL((scan_carry_kernel<NM>), dim3(n_seg, cb), dim3(128), 0, s, A, state, seg_pos0, seg_slot,   \
+                       seg_chunk0, cs, csd, C, N);                                                                \
+    K8S_SCAN_M(NM, 2, n_chunks);                                                                                  \
+  }
   if (N <= 16) {
-    K8S_SCAN(16);
+    K8S_SCAN(16)
   } else if (N <= 32) {
-    K8S_SCAN(32);
+    K8S_SCAN(32)
   } else if (N <= 64) {
-    K8S_SCAN(64);
+    K8S_SCAN(64)
   } else {
-    K8S_SCAN(128);
+    K8S_SCAN(128)
   }
 #undef K8S_SCAN
+#undef K8S_SCAN_M
   return (int)hipGetLastError();
 }
 
-K8S_API int k8s_retention(const float* qkvg, int qs, const int* positions, const float* decay, float* state,
+K8S_API int k8s_retention(float* qkvg, int qs, const int* positions, const float* decay, float* state,
                           const int* seg_row0, const int* seg_pos0, const int* seg_slot, void* out, int n_seg, int H,
-                          int D, int V, int rot, float base, float eps, int odt, hipStream_t s) {
-  if (n_seg <= 0) return 0;
-  if (V < 1 || V > 256 || rot < 0 || rot > D || (rot & 1) || rot / 2 > 256) return (int)hipErrorInvalidValue;
-  const int NDG = 256 / V;
+                          int D, int V, int rot, float base, float eps, int odt, hipStream_t s, int T, float* oraw) {
+  if (n_seg <= 0 || T <= 0) return 0;
+  if (V < 1 || rot < 0 || rot > D || (rot & 1)) return (int)hipErrorInvalidValue;
+  const int VBS = V < 64 ? V : 64, NDG = 256 / VBS;
   if ((D + NDG - 1) / NDG > kRetDpt) return (int)hipErrorInvalidValue;
-  const size_t lds = (size_t)(2 * D + V + NDG * V + rot) * sizeof(float);
-  K8S_MDT(odt, hipLaunchKernelGGL((retention_kernel<TA>), dim3(n_seg, H), dim3(256), lds, s, qkvg, qs, positions,
-                                  decay, state, seg_row0, seg_pos0, seg_slot, (TA*)out, H, D, V, rot, base, eps));
+  const size_t lds = (size_t)kRetTb * (2 * D + VBS + NDG * VBS) * sizeof(float);
+  if (lds > 64 * 1024 || (size_t)rot * sizeof(float) > 64 * 1024) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(retention_rope_kernel, dim3(T), dim3(256), rot * sizeof(float) + 8, s, qkvg, qs, positions, H, D,
+                     rot, base);
+  if (lds > 48 * 1024 &&
+      hipFuncSetAttribute((const void*)retention_scan_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
+    return (int)hipGetLastError();
+  hipLaunchKernelGGL(retention_scan_kernel, dim3(n_seg, H, (V + VBS - 1) / VBS), dim3(256), lds, s, qkvg, qs, decay,
+                     state, seg_row0, seg_pos0, seg_slot, oraw, H, D, V, VBS);
+  const int n_rh = T * H;
+  K8S_MDT(odt, hipLaunchKernelGGL((head_norm_gate_kernel<TA>), dim3((n_rh + 3) / 4), dim3(256), 0, s, oraw,
+                                  qkvg + 2 * H * D + H * V, qs, (TA*)out, n_rh, H, V, eps));
   return (int)hipGetLastError();
 }

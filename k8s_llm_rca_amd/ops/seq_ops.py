@@ -80,6 +80,28 @@ class SegMeta:
             got = self._items[key] = host.to(self.row_seg.device, non_blocking=True)
         return got
 
+    def chunk_ranges(self, rows: int, min_rows: int) -> Optional[tuple]:
+        """Segments cut into chunks of at most ``rows`` rows, for recurrences that run the chunks in
+        parallel: (chunks [n, 4] int32: segment, first row, rows, 0; seg_chunk0 [n_seg + 1] int32), both on
+        the device; None when no segment has more than ``min_rows`` rows (the sequential kernel runs)."""
+        key = ("ranges", rows, min_rows)
+        if key in self._items:
+            return self._items[key]
+        out = None
+        if max(b - a for a, b in zip(self.row0_host[:-1], self.row0_host[1:])) > min_rows:
+            ch, c0 = [], [0]
+            for s in range(self.n_seg):
+                a, b = self.row0_host[s], self.row0_host[s + 1]
+                ch += [(s, r, min(rows, b - r), 0) for r in range(a, b, rows)]
+                c0.append(len(ch))
+            host = torch.from_numpy(np.asarray([v for c in ch for v in c] + c0, dtype=np.int32))
+            if self.row_seg.device.type == "cuda":
+                host = host.pin_memory()
+            dev = host.to(self.row_seg.device, non_blocking=True)
+            out = (dev[:4 * len(ch)].view(-1, 4), dev[4 * len(ch):])
+        self._items[key] = out
+        return out
+
     def scan_chunks(self, rows: int) -> Optional[torch.Tensor]:
         """Chunks of at most ``rows`` rows for the time-parallel recurrence ([n, 4] int32 on the device:
         segment, first row, rows, index of the segment's first chunk); None when no segment is longer
@@ -102,6 +124,7 @@ class SegMeta:
 
 
 SCAN_CHUNK = 64     # rows per chunk of the time-parallel minGRU
+SSM_CHUNK = 64      # rows per chunk of the time-parallel selective scan
 
 
 def _dt(t: torch.dtype) -> int:
@@ -382,10 +405,19 @@ def selective_scan(xc: torch.Tensor, dtp: torch.Tensor, dt_bias: torch.Tensor, d
         assert dbc.dtype == torch.float32 and dbc.stride(1) == 1 and dbc.shape[1] >= R + 2 * N
         assert z.stride(1) == 1 and z.dtype == xc.dtype and state.is_contiguous() and state.shape[1:] == (C, N)
         assert A.dtype == D.dtype == dt_bias.dtype == torch.float32 and A.is_contiguous()
+        # long portions: chunks run in parallel (a pass from zero states, a carry over the chunks, the
+        # chunks again from their start states); short ones token by token
+        cr = seg.chunk_ranges(SSM_CHUNK, 2 * SSM_CHUNK)
+        chunks, c0, cs, csd, nch = None, None, None, None, 0
+        if cr is not None:
+            chunks, c0 = cr
+            nch = chunks.shape[0]
+            cs = scratch(nch * C * N, torch.float32, xc.device)
+            csd = scratch(nch * C, torch.float32, xc.device)
         check(lib().k8s_selective_scan(ptr(xc), _dt(xc.dtype), ptr(dtp), ptr(dt_bias), ptr(dbc), dbc.stride(0), R,
                                        ptr(A), ptr(D), ptr(z), z.stride(0), ptr(state), ptr(seg.seg_row0),
                                        ptr(seg.seg_pos0), ptr(seg.seg_slot), ptr(y), seg.n_seg, C, N, T,
-                                       stream_ptr(xc)), "selective_scan")
+                                       stream_ptr(xc), ptr(chunks), nch, ptr(c0), ptr(cs), ptr(csd)), "selective_scan")
         return y
     dt = torch.nn.functional.softplus(dtp + dt_bias)
     xf, zf = xc.float(), z.float()
@@ -405,15 +437,18 @@ def retention(qkvg: torch.Tensor, H: int, D: int, V: int, decay: torch.Tensor, r
     """Retention per head, fp32: rows of ``qkvg`` [T, 2HD + 2HV] fp32 = (q | k | v | g).  q and k are
     rotated on their first ``rot_dims`` entries (entry i paired with i + rot_dims / 2, angle
     ``pos * rot_base^(-2i / rot_dims)``), k is scaled by ``D^(-1/2)``; ``S <- decay_h S + k v^T``;
-    ``o = S^T q``; the result is ``o / rms(o) * silu(g)`` [T, H * V].  ``state`` [slots, H, D, V] fp32."""
+    ``o = S^T q``; the result is ``o / rms(o) * silu(g)`` [T, H * V].  ``state`` [slots, H, D, V] fp32.
+    On the device q and k are rotated IN PLACE in ``qkvg``."""
     T = qkvg.shape[0]
     out = torch.empty(T, H * V, dtype=out_dtype, device=qkvg.device)
     if use_hip(qkvg):
         assert qkvg.dtype == torch.float32 and qkvg.stride(1) == 1 and qkvg.shape[1] == 2 * H * (D + V)
         assert state.is_contiguous() and state.shape[1:] == (H, D, V) and decay.dtype == torch.float32
+        oraw = scratch(T * H * V, torch.float32, qkvg.device)
         check(lib().k8s_retention(ptr(qkvg), qkvg.stride(0), ptr(positions), ptr(decay), ptr(state), ptr(seg.seg_row0),
                                   ptr(seg.seg_pos0), ptr(seg.seg_slot), ptr(out), seg.n_seg, H, D, V, rot_dims,
-                                  float(rot_base), float(eps), _dt(out_dtype), stream_ptr(qkvg)), "retention")
+                                  float(rot_base), float(eps), _dt(out_dtype), stream_ptr(qkvg), T, ptr(oraw)),
+              "retention")
         return out
     half = rot_dims // 2
     f = torch.exp(-(2.0 * torch.arange(half, dtype=torch.float64) / max(rot_dims, 1)) * math.log(rot_base))

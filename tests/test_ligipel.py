@@ -327,7 +327,8 @@ def test_selective_scan_across_portions(backend, C, Ns, R):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("H,D,V,rot", [(3, 8, 12, 8), (2, 12, 4, 6), (1, 4, 4, 0), (4, 32, 64, 32), (2, 64, 128, 16)])
+@pytest.mark.parametrize("H,D,V,rot", [(3, 8, 12, 8), (2, 12, 4, 6), (1, 4, 4, 0), (4, 32, 64, 32), (2, 64, 128, 16),
+                                       (2, 16, 100, 10), (1, 128, 256, 128)])
 def test_retention_across_portions_and_slots(backend, H, D, V, rot):
     dev, dt = backend
     T, eps, base = 29, 1e-5, 500.0
@@ -339,9 +340,9 @@ def test_retention_across_portions_and_slots(backend, H, D, V, rot):
     k = O.rotate(qkvg[:, H * D:2 * H * D].reshape(T, H, D), pos, rot, base, DT) * D ** -0.5
     v = qkvg[:, 2 * H * D:2 * H * D + H * V].reshape(T, H, V)
     o = O.rms(O.retention_core(q, k, v, decay), eps).reshape(T, H * V) * F.silu(qkvg[:, 2 * H * D + H * V:])
-    qd = qkvg.float().to(dev)
     dec = torch.tensor(decay, dtype=torch.float32, device=dev)
-    for cuts in [(T,), (1, 2, 1, 10), (7, 1, 1)]:
+    for cuts in [(T,), (1, 2, 1, 10), (7, 1, 1), (17, 2)]:
+        qd = qkvg.float().to(dev)                           # the device kernels rotate q and k in place
         state = torch.full((3, H, D, V), float("nan"), device=dev)
         first = [True]
 
@@ -351,6 +352,43 @@ def test_retention_across_portions_and_slots(backend, H, D, V, rot):
             p = torch.arange(pos0 + a, pos0 + e, dtype=torch.int32, device=dev)
             return S.retention(qd[a:e], H, D, V, dec, rot, base, state, sg, p, eps, dt)
         close(in_portions(run, T, cuts), o, dt, scale=4.0)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_selective_scan_long_portions_parallel_over_time(backend):
+    """Portions long enough for the chunk-parallel kernels, beside a short one in the same step, and a
+    sequence that goes on from a long portion token by token."""
+    dev, dt = backend
+    T, C, Ns, R = 520, 48, 8, 4
+    xc = rnd(T, C, seed=1).to(torch.bfloat16).double()
+    z = rnd(T, 2 * C, seed=2).to(torch.bfloat16).double()
+    dtp, bias = rnd(T, C, seed=3), rnd(C, seed=4) - 1.0
+    dbc = rnd(T, R + 2 * Ns, seed=5)
+    A, D = -torch.exp(rnd(C, Ns, seed=6, std=0.5)), rnd(C, seed=7)
+
+    def plain(a, e):
+        return (O.selective_scan(xc[a:e], F.softplus(dtp[a:e] + bias), A, dbc[a:e, R:R + Ns], dbc[a:e, R + Ns:], D)
+                * F.silu(z[a:e, C:]))
+    f32 = lambda t: t.float().to(dev)  # noqa: E731
+    xd, zd = xc.to(dev).to(dt), z.to(dev).to(dt)
+    state = torch.full((3, C, Ns), float("nan"), device=dev)
+
+    def run(a, e, sg):
+        return S.selective_scan(xd[a:e].contiguous(), f32(dtp[a:e]), f32(bias), f32(dbc[a:e]), R, f32(A), f32(D),
+                                zd[a:e, C:], state, sg)
+    # rows 0..299: sequence X; rows 300..519: sequence Y
+    o1 = run(0, 200, seg_meta([200], [0], [0], dev))
+    oy = run(300, 305, seg_meta([5], [0], [2], dev))
+    got_x = torch.cat([o1, run(200, 201, seg_meta([1], [200], [0], dev)),
+                       run(201, 300, seg_meta([99], [201], [0], dev))])
+    close(got_x, plain(0, 300), dt, scale=4.0)
+    # one step with two segments: Y goes on with 215 rows (chunked) beside the first 3 rows of another sequence
+    xs = torch.cat([xd[305:520], xd[0:3]]).contiguous()
+    both = S.selective_scan(xs, f32(torch.cat([dtp[305:520], dtp[0:3]])), f32(bias),
+                            f32(torch.cat([dbc[305:520], dbc[0:3]])), R, f32(A), f32(D),
+                            torch.cat([zd[305:520], zd[0:3]])[:, C:], state, seg_meta([215, 3], [5, 0], [2, 1], dev))
+    close(torch.cat([oy, both[:215]]), plain(300, 520), dt, scale=4.0)
+    close(both[215:], plain(0, 3), dt, scale=4.0)
 
 
 def paged(x, block_size, order, dev, dt):
