@@ -27,6 +27,15 @@ __device__ __forceinline__ void stm<uint16_t>(uint16_t* p, size_t i, float v) { 
 
 __device__ __forceinline__ float silu_f(float v) { return v / (1.f + expf(-v)); }
 
+// exp of the recurrence's decays: the full-precision routine where activations are fp32, the hardware
+// exponential (exp2 of x log2 e, about 1e-6 relative) where they are bf16
+template <typename TA>
+__device__ __forceinline__ float decay_exp(float x);
+template <>
+__device__ __forceinline__ float decay_exp<float>(float x) { return expf(x); }
+template <>
+__device__ __forceinline__ float decay_exp<uint16_t>(float x) { return __expf(x); }
+
 // out[r][c] = act(b[c] + sum_j w[c][j] * in(r - (taps - 1 - j))): the last column is the current
 // token's tap.  Inputs before the segment come from the slot's tail (entry k = the input at
 // position pos0 - (taps - 1) + k), zeros before the sequence.  x rows have stride xs.
@@ -145,7 +154,7 @@ __global__ void __launch_bounds__(128) selective_scan_kernel(const TA* __restric
 #pragma unroll
     for (int n = 0; n < NMAX; ++n)
       if (n < N) {
-        S[n] = fmaf(expf(dt * Ac[n]), S[n], dx * Bp[n]);
+        S[n] = fmaf(decay_exp<TA>(dt * Ac[n]), S[n], dx * Bp[n]);
         if (MODE != 1) acc = fmaf(S[n], Cp[n], acc);
       }
     if (MODE != 1) {
@@ -200,7 +209,7 @@ __global__ void __launch_bounds__(128) scan_carry_kernel(const float* __restrict
 //   1. retention_rope_kernel (one workgroup per token, in place): q and k are rotated on their first
 //      `rot` entries (entry i with i + rot / 2; angle = pos * base^(-2 i / rot), formed in double) and k is
 //      scaled by D^(-1/2);
-//   2. retention_scan_kernel, one workgroup per (segment, head, block of <= 64 value columns), tokens
+//   2. retention_scan_kernel, one workgroup per (segment, head, block of <= 32 value columns), tokens
 //      in batches of 16 through LDS:  S <- decay S + k v^T;  o = S^T q  (fp32, written raw).
 //      Thread (dg, v) of NDG x VBS owns S[d][v] for d = dg, dg + NDG, ...  state [slots][H][D][V];
 //   3. head_norm_gate_kernel: out = o / rms(o over the head's V) * silu(g).
@@ -232,16 +241,22 @@ __global__ void __launch_bounds__(256) retention_rope_kernel(float* __restrict__
   }
 }
 
-constexpr int kRetDpt = 64;   // state rows per thread
 constexpr int kRetTb = 16;    // tokens per batch
+// MODE 0: blockIdx.x = segment, from the slot's state (or zero at position 0) to the slot's state.
+// Long segments are cut into chunks ([n][4]: segment, first row, rows, -) that run in parallel:
+// MODE 1: a chunk from a zero state, its end state goes to cs [chunks][H][D][V], no output;
+// (retention_carry_kernel then turns cs into every chunk's START state and advances the slot's state)
+// MODE 2: the chunk again from its start state, writing o.
+template <int DPT, int MODE>
 __global__ void __launch_bounds__(256) retention_scan_kernel(const float* __restrict__ qkvg, int qs,
                                                              const float* __restrict__ decay, float* __restrict__ state,
                                                              const int* __restrict__ seg_row0,
                                                              const int* __restrict__ seg_pos0,
                                                              const int* __restrict__ seg_slot, float* __restrict__ oraw,
-                                                             int H, int D, int V, int VBS) {
+                                                             int H, int D, int V, int VBS,
+                                                             const int* __restrict__ chunks, float* __restrict__ cs) {
   extern __shared__ float sm[];
-  const int sg = blockIdx.x, hh = blockIdx.y, v0 = blockIdx.z * VBS, tid = threadIdx.x;
+  const int it = blockIdx.x, hh = blockIdx.y, v0 = blockIdx.z * VBS, tid = threadIdx.x;
   const int NDG = 256 / VBS;
   float* sq = sm;                          // [TB][D]
   float* sk = sq + kRetTb * D;             // [TB][D]
@@ -249,13 +264,24 @@ __global__ void __launch_bounds__(256) retention_scan_kernel(const float* __rest
   float* part = sv + kRetTb * VBS;         // [TB][NDG][VBS]
   const int v = tid % VBS, dg = tid / VBS;
   const bool own = dg < NDG && v0 + v < V;
-  const int r0 = seg_row0[sg], r1 = seg_row0[sg + 1];
-  const bool fresh = seg_pos0[sg] == 0;
-  float* st = state + ((size_t)seg_slot[sg] * H + hh) * D * V + v0;
+  int r0, r1;
+  bool fresh;
+  float* st;
+  if (MODE == 0) {
+    r0 = seg_row0[it];
+    r1 = seg_row0[it + 1];
+    fresh = seg_pos0[it] == 0;
+    st = state + ((size_t)seg_slot[it] * H + hh) * D * V + v0;
+  } else {
+    r0 = chunks[it * 4 + 1];
+    r1 = r0 + chunks[it * 4 + 2];
+    fresh = MODE == 1;
+    st = cs + ((size_t)it * H + hh) * D * V + v0;
+  }
   const float dec = decay[hh];
-  float S[kRetDpt];
+  float S[DPT];
 #pragma unroll
-  for (int i = 0; i < kRetDpt; ++i) {
+  for (int i = 0; i < DPT; ++i) {
     const int d = dg + i * NDG;
     S[i] = (own && d < D && !fresh) ? st[(size_t)d * V + v] : 0.f;
   }
@@ -280,31 +306,60 @@ __global__ void __launch_bounds__(256) retention_scan_kernel(const float* __rest
         const float* qq = sq + tb * D;
         float acc = 0.f;
 #pragma unroll
-        for (int i = 0; i < kRetDpt; ++i) {
+        for (int i = 0; i < DPT; ++i) {
           const int d = dg + i * NDG;
           if (d < D) {
             S[i] = fmaf(dec, S[i], kq[d] * vv);
-            acc = fmaf(S[i], qq[d], acc);
+            if (MODE != 1) acc = fmaf(S[i], qq[d], acc);
           }
         }
-        part[(tb * NDG + dg) * VBS + v] = acc;
+        if (MODE != 1) part[(tb * NDG + dg) * VBS + v] = acc;
       }
     }
-    __syncthreads();
-    for (int e = tid; e < nb * VBS; e += 256) {
-      const int tb = e / VBS, vv = e - tb * VBS;
-      if (v0 + vv < V) {
-        float o = 0.f;
-        for (int g = 0; g < NDG; ++g) o += part[(tb * NDG + g) * VBS + vv];
-        oraw[(size_t)(t0 + tb) * H * V + hh * V + v0 + vv] = o;
+    if (MODE != 1) {
+      __syncthreads();
+      for (int e = tid; e < nb * VBS; e += 256) {
+        const int tb = e / VBS, vv = e - tb * VBS;
+        if (v0 + vv < V) {
+          float o = 0.f;
+          for (int g = 0; g < NDG; ++g) o += part[(tb * NDG + g) * VBS + vv];
+          oraw[(size_t)(t0 + tb) * H * V + hh * V + v0 + vv] = o;
+        }
       }
     }
   }
+  if (MODE != 2) {
 #pragma unroll
-  for (int i = 0; i < kRetDpt; ++i) {
-    const int d = dg + i * NDG;
-    if (own && d < D) st[(size_t)d * V + v] = S[i];
+    for (int i = 0; i < DPT; ++i) {
+      const int d = dg + i * NDG;
+      if (own && d < D) st[(size_t)d * V + v] = S[i];
+    }
   }
+}
+
+// Between the two chunk passes, one thread per state entry of a (segment, head): walk the segment's
+// chunks, replace every chunk's end-from-zero state by its START state, leave the final state in the slot.
+__global__ void __launch_bounds__(256) retention_carry_kernel(const float* __restrict__ decay, float* __restrict__ state,
+                                                              const int* __restrict__ seg_pos0,
+                                                              const int* __restrict__ seg_slot,
+                                                              const int* __restrict__ seg_chunk0,
+                                                              const int* __restrict__ chunks, float* __restrict__ cs,
+                                                              int H, int DV) {
+  const int sg = blockIdx.x, hh = blockIdx.y, e = blockIdx.z * 256 + threadIdx.x;
+  if (e >= DV) return;
+  float* st = state + ((size_t)seg_slot[sg] * H + hh) * DV + e;
+  float S = seg_pos0[sg] == 0 ? 0.f : *st;
+  const float dec = decay[hh];
+  for (int k = seg_chunk0[sg]; k < seg_chunk0[sg + 1]; ++k) {
+    float* ck = cs + ((size_t)k * H + hh) * DV + e;
+    const int n = chunks[k * 4 + 2];
+    float p = 1.f;
+    for (int i = 0; i < n; ++i) p *= dec;
+    const float loc = *ck;
+    *ck = S;
+    S = fmaf(p, S, loc);
+  }
+  *st = S;
 }
 
 // out[r][h] = o / sqrt(mean(o^2 over V) + eps) * silu(g): one wave per (row, head).
@@ -389,20 +444,47 @@ K8S_API int k8s_selective_scan(const void* xc, int dt, const float* dtp, const f
 
 K8S_API int k8s_retention(float* qkvg, int qs, const int* positions, const float* decay, float* state,
                           const int* seg_row0, const int* seg_pos0, const int* seg_slot, void* out, int n_seg, int H,
-                          int D, int V, int rot, float base, float eps, int odt, hipStream_t s, int T, float* oraw) {
+                          int D, int V, int rot, float base, float eps, int odt, hipStream_t s, int T, float* oraw,
+                          const int* chunks, int n_chunks, const int* seg_chunk0, float* cs) {
   if (n_seg <= 0 || T <= 0) return 0;
   if (V < 1 || rot < 0 || rot > D || (rot & 1)) return (int)hipErrorInvalidValue;
-  const int VBS = V < 64 ? V : 64, NDG = 256 / VBS;
-  if ((D + NDG - 1) / NDG > kRetDpt) return (int)hipErrorInvalidValue;
+  const int VBS = V < 32 ? V : 32, NDG = 256 / VBS, dpt = (D + NDG - 1) / NDG;
+  if (dpt > 64) return (int)hipErrorInvalidValue;
   const size_t lds = (size_t)kRetTb * (2 * D + VBS + NDG * VBS) * sizeof(float);
-  if (lds > 64 * 1024 || (size_t)rot * sizeof(float) > 64 * 1024) return (int)hipErrorInvalidValue;
+  if (lds > 160 * 1024 || (size_t)rot * sizeof(float) > 64 * 1024) return (int)hipErrorInvalidValue;
   hipLaunchKernelGGL(retention_rope_kernel, dim3(T), dim3(256), rot * sizeof(float) + 8, s, qkvg, qs, positions, H, D,
                      rot, base);
-  if (lds > 48 * 1024 &&
-      hipFuncSetAttribute((const void*)retention_scan_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
-    return (int)hipGetLastError();
-  hipLaunchKernelGGL(retention_scan_kernel, dim3(n_seg, H, (V + VBS - 1) / VBS), dim3(256), lds, s, qkvg, qs, decay,
-                     state, seg_row0, seg_pos0, seg_slot, oraw, H, D, V, VBS);
+  const int vb = (V + VBS - 1) / VBS;
+#define K8S_RET_M(DP, MODE, items)                                                                              \
+  {                                                                                                             \
+    auto k = retention_scan_kernel<DP, MODE>;                                                                   \
+    if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) \
+      return (int)hipGetLastError();                                                                            \
+    hipLaunchKernelGGL(k, dim3(items, H, vb), dim3(256), lds, s, qkvg, qs, decay, state, seg_row0, seg_pos0,    \
+                       seg_slot, oraw, H, D, V, VBS, chunks, cs);                                               \
+  }
+#define K8S_RET(DP)                                                                                             \
+  if (chunks == nullptr) {                                                                                      \
+    K8S_RET_M(DP, 0, n_seg)                                                                                     \
+  } else {                                                                                                      \
+    K8S_RET_M(DP, 1, n_chunks)                                                                                  \
+    hipLaunchKernelGGL(retention_carry_kernel, dim3(n_seg, H, (D * V + 255) / 256), dim3(256), 0, s, decay, state, \
+                       seg_pos0, seg_slot, seg_chunk0, chunks, cs, H, D * V);                                   \
+    K8S_RET_M(DP, 2, n_chunks)                                                                                  \
+  }
+  if (dpt <= 4) {
+    K8S_RET(4)
+  } else if (dpt <= 8) {
+    K8S_RET(8)
+  } else if (dpt <= 16) {
+    K8S_RET(16)
+  } else if (dpt <= 32) {
+    K8S_RET(32)
+  } else {
+    K8S_RET(64)
+  }
+#undef K8S_RET
+#undef K8S_RET_M
   const int n_rh = T * H;
   K8S_MDT(odt, hipLaunchKernelGGL((head_norm_gate_kernel<TA>), dim3((n_rh + 3) / 4), dim3(256), 0, s, oraw,
                                   qkvg + 2 * H * D + H * V, qs, (TA*)out, n_rh, H, V, eps));

@@ -124,7 +124,7 @@ class SegMeta:
 
 
 SCAN_CHUNK = 64     # rows per chunk of the time-parallel minGRU
-SSM_CHUNK = 64      # rows per chunk of the time-parallel selective scan
+SSM_CHUNK = 64      # rows per chunk of the time-parallel selective scan and retention
 
 
 def _dt(t: torch.dtype) -> int:
@@ -445,10 +445,18 @@ def retention(qkvg: torch.Tensor, H: int, D: int, V: int, decay: torch.Tensor, r
         assert qkvg.dtype == torch.float32 and qkvg.stride(1) == 1 and qkvg.shape[1] == 2 * H * (D + V)
         assert state.is_contiguous() and state.shape[1:] == (H, D, V) and decay.dtype == torch.float32
         oraw = scratch(T * H * V, torch.float32, qkvg.device)
+        # long portions: chunks in parallel (end states from zero, a carry over the chunks, the chunks
+        # again from their start states); short ones token by token
+        cr = seg.chunk_ranges(SSM_CHUNK, 2 * SSM_CHUNK)
+        chunks, c0, cs, nch = None, None, None, 0
+        if cr is not None:
+            chunks, c0 = cr
+            nch = chunks.shape[0]
+            cs = scratch(nch * H * D * V, torch.float32, qkvg.device)
         check(lib().k8s_retention(ptr(qkvg), qkvg.stride(0), ptr(positions), ptr(decay), ptr(state), ptr(seg.seg_row0),
                                   ptr(seg.seg_pos0), ptr(seg.seg_slot), ptr(out), seg.n_seg, H, D, V, rot_dims,
-                                  float(rot_base), float(eps), _dt(out_dtype), stream_ptr(qkvg), T, ptr(oraw)),
-              "retention")
+                                  float(rot_base), float(eps), _dt(out_dtype), stream_ptr(qkvg), T, ptr(oraw),
+                                  ptr(chunks), nch, ptr(c0), ptr(cs)), "retention")
         return out
     half = rot_dims // 2
     f = torch.exp(-(2.0 * torch.arange(half, dtype=torch.float64) / max(rot_dims, 1)) * math.log(rot_base))

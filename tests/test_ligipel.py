@@ -391,6 +391,34 @@ def test_selective_scan_long_portions_parallel_over_time(backend):
     close(both[215:], plain(0, 3), dt, scale=4.0)
 
 
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("H,D,V", [(2, 8, 12), (3, 32, 64), (2, 64, 128)])
+def test_retention_long_portions_parallel_over_time(backend, H, D, V):
+    """Portions long enough for the chunk-parallel kernels, then on token by token, beside another sequence."""
+    dev, dt = backend
+    T, eps, base, rot = 330, 1e-5, 1e4, D
+    qkvg = rnd(T, 2 * H * (D + V), seed=H + D)
+    decay = [1.0 - 2.0 ** (-4 - h) for h in range(H)]
+    pos = torch.arange(T)
+    q = O.rotate(qkvg[:, :H * D].reshape(T, H, D), pos, rot, base, DT)
+    k = O.rotate(qkvg[:, H * D:2 * H * D].reshape(T, H, D), pos, rot, base, DT) * D ** -0.5
+    v = qkvg[:, 2 * H * D:2 * H * D + H * V].reshape(T, H, V)
+    want = O.rms(O.retention_core(q, k, v, decay), eps).reshape(T, H * V) * F.silu(qkvg[:, 2 * H * D + H * V:])
+    dec = torch.tensor(decay, dtype=torch.float32, device=dev)
+    state = torch.full((3, H, D, V), float("nan"), device=dev)
+
+    def run(rows, sg, p):
+        return S.retention(qkvg[rows].float().to(dev), H, D, V, dec, rot, base, state, sg,
+                           torch.tensor(p, dtype=torch.int32, device=dev), eps, dt)
+    # one step: rows 0..199 of the sequence (slot 1) beside rows 0..2 of the same tokens as another one (slot 0)
+    rows = list(range(200)) + [0, 1, 2]
+    o1 = run(rows, seg_meta([200, 3], [0, 0], [1, 0], dev), list(range(200)) + [0, 1, 2])
+    close(o1[200:], want[:3], dt, scale=4.0)
+    o2 = run([200], seg_meta([1], [200], [1], dev), [200])
+    o3 = run(list(range(201, 330)), seg_meta([129], [201], [1], dev), list(range(201, 330)))
+    close(torch.cat([o1[:200], o2, o3]), want, dt, scale=4.0)
+
+
 def paged(x, block_size, order, dev, dt):
     """Rows of ``x`` [n, w] laid into pages in ``order``; returns (pages [nb, BS, w], block table row)."""
     n, w = x.shape
