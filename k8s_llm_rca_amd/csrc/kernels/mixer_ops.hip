@@ -27,14 +27,21 @@ __device__ __forceinline__ void stm<uint16_t>(uint16_t* p, size_t i, float v) { 
 
 __device__ __forceinline__ float silu_f(float v) { return v / (1.f + expf(-v)); }
 
-// exp of the recurrence's decays: the full-precision routine where activations are fp32, the hardware
-// exponential (exp2 of x log2 e, about 1e-6 relative) where they are bf16
+// exp of the recurrence's decays (arguments <= 0): the full-precision routine where activations are
+// fp32; where they are bf16 the hardware exponential 2^x (about 1e-6 relative, tiny results flush to 0)
+// with log2(e) folded into A beforehand
 template <typename TA>
-__device__ __forceinline__ float decay_exp(float x);
+struct DecayExp;
 template <>
-__device__ __forceinline__ float decay_exp<float>(float x) { return expf(x); }
+struct DecayExp<float> {
+  static constexpr float kPre = 1.f;
+  static __device__ __forceinline__ float f(float x) { return expf(x); }
+};
 template <>
-__device__ __forceinline__ float decay_exp<uint16_t>(float x) { return __expf(x); }
+struct DecayExp<uint16_t> {
+  static constexpr float kPre = 1.4426950408889634f;
+  static __device__ __forceinline__ float f(float x) { return __builtin_amdgcn_exp2f(x); }
+};
 
 // out[r][c] = act(b[c] + sum_j w[c][j] * in(r - (taps - 1 - j))): the last column is the current
 // token's tap.  Inputs before the segment come from the slot's tail (entry k = the input at
@@ -137,7 +144,7 @@ __global__ void __launch_bounds__(128) selective_scan_kernel(const TA* __restric
   float S[NMAX], Ac[NMAX];
 #pragma unroll
   for (int n = 0; n < NMAX; ++n) {
-    Ac[n] = n < N ? A[(size_t)c * N + n] : 0.f;
+    Ac[n] = n < N ? A[(size_t)c * N + n] * DecayExp<TA>::kPre : 0.f;
     S[n] = (n < N && !fresh) ? st[n] : 0.f;
   }
   const float Dc = Dp[c], bias = dt_bias[c];
@@ -154,7 +161,7 @@ __global__ void __launch_bounds__(128) selective_scan_kernel(const TA* __restric
 #pragma unroll
     for (int n = 0; n < NMAX; ++n)
       if (n < N) {
-        S[n] = fmaf(decay_exp<TA>(dt * Ac[n]), S[n], dx * Bp[n]);
+        S[n] = fmaf(DecayExp<TA>::f(dt * Ac[n]), S[n], dx * Bp[n]);
         if (MODE != 1) acc = fmaf(S[n], Cp[n], acc);
       }
     if (MODE != 1) {

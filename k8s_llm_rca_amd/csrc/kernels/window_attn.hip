@@ -178,6 +178,8 @@ struct WinArgs {
 };
 
 __device__ __forceinline__ bf16x8 wld16(const uint16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+// 2^x on the hardware exponential; the arguments here are <= 0 or -inf (results in [0, 1], tiny ones flush to 0)
+__device__ __forceinline__ float wexp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 template <int NDC>
 __device__ __forceinline__ void win_scores(const bf16x8 (&kf)[2][NDC], const bf16x8 (&qf)[NDC], int kb, int hq,
@@ -262,8 +264,8 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(WinArgs a) {
         const float mn = fmaxf(m2[hh], cmax);
         float ps = 0.f;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) ps += exp2f(p[j] - mn);
-        l[hh] = l[hh] * exp2f(m2[hh] - mn) + ps;
+        for (int j = 0; j < 8; ++j) ps += wexp2(p[j] - mn);
+        l[hh] = l[hh] * wexp2(m2[hh] - mn) + ps;
         m2[hh] = mn;
       }
     }
@@ -273,7 +275,7 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(WinArgs a) {
     float lt = l[hh];
     lt += __shfl_xor(lt, 16, 64);
     lt += __shfl_xor(lt, 32, 64);
-    inv_l[hh] = 1.f / (lt + exp2f(-m2[hh]));     // + the sink
+    inv_l[hh] = 1.f / (lt + wexp2(-m2[hh]));     // + the sink
   }
   // ---- pass 2: weights, mixed over heads, times the values
   f32x4 o[HW][NV];
@@ -309,7 +311,7 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(WinArgs a) {
           for (int t = 0; t < 2; ++t) {
             f32x4 e;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) e[i] = exp2f(p[4 * t + i] - m2[hh]) * inv_l[hh];
+            for (int i = 0; i < 4; ++i) e[i] = wexp2(p[4 * t + i] - m2[hh]) * inv_l[hh];
             *reinterpret_cast<f32x4*>(Ph + t * 256) = e;
           }
         }

@@ -36,7 +36,7 @@ import torch
 from ..ops import moe as M
 from ..ops import norm as N
 from ..ops import seq_ops as S
-from ..ops.linear import linear, linear_f32out
+from ..ops.linear import linear, linear_f32out, swiglu_gemm
 from ..parallel.groups import ParallelContext, single
 
 RENORM_EPS = 1e-20      # router: chosen scores are divided by their sum + RENORM_EPS
@@ -379,12 +379,21 @@ class LigipelModel:
                                 renorm_eps=RENORM_EPS)
         order, inv, offsets = M.align(ids, f.experts)
         xp = M.gather_rows(h, order, f.top)
-        act = M.glu_clamp(M.grouped_auto(xp, L["w13"], offsets), 1.0, math.inf, 0.0)      # silu(gate) * up
+        rows, W = xp.shape
+        if (xp.is_cuda and xp.dtype == torch.bfloat16 and rows > M.BIG_MIN_ROWS and M.grouped_big_ok(rows, f.ff, W, True)
+                and M.grouped_big_ok(rows, W, f.ff, False)):
+            # prefill sizes: the grouped MFMA GEMM with the gated unit in its epilogue (gate_up never written)
+            act = M.grouped_big(xp, L["w13"], offsets, silu=True)
+        else:
+            act = M.glu_clamp(M.grouped_auto(xp, L["w13"], offsets), 1.0, math.inf, 0.0)  # silu(gate) * up
         yp = M.grouped_auto(act, L["w2"], offsets)
         routed = M.combine_f32(yp, inv, T, f.top, w)
         shared = None
         if f.shared_ff:
-            shared = self._lin32(M.glu_clamp(linear(h, L["ws13"]), 1.0, math.inf, 0.0), L["ws2"])
+            act = swiglu_gemm(h, L["ws13"])                       # one launch where a fused kernel takes the shape
+            if act is None:
+                act = M.glu_clamp(linear(h, L["ws13"]), 1.0, math.inf, 0.0)
+            shared = self._lin32(act, L["ws2"])
         return routed, shared
 
     def forward(self, inp: S.SegStepInputs, kcs: List[torch.Tensor], vcs: List[torch.Tensor],
