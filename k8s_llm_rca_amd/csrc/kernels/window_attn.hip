@@ -150,7 +150,7 @@ __global__ void __launch_bounds__(256) window_attn_rows_kernel(const TA* __restr
 
 
 // ---------------------------------------------------------------------------------------------
-// Matrix-core form (bf16, v_mfma_f32_16x16x32_bf16).  A workgroup of four waves owns a tile of up
+// Matrix-core form (bf16, v_mfma_f32_16x16x32_bf16).  A workgroup of ceil(H / HW) waves owns a tile of up
 // to 16 consecutive tokens of one segment; wave w owns the heads w HW .. w HW + HW - 1.  Keys go
 // in blocks of 32 (never across a page: BS % 32 == 0).  Swapped QK^T as in the other attention
 // kernels: a lane owns ONE query (lane & 15) and, per block, the scores of keys 8 q .. 8 q + 7 of its
@@ -201,7 +201,7 @@ __device__ __forceinline__ void win_scores(const bf16x8 (&kf)[2][NDC], const bf1
 }
 
 template <int NDC, int NV, int HW>
-__global__ void __launch_bounds__(256) window_attn_mfma_kernel(WinArgs a) {
+__global__ void __launch_bounds__(512) window_attn_mfma_kernel(WinArgs a) {
   constexpr int D = NDC * 32, V = NV * 16;
   constexpr float kLog2e = 1.4426950408889634f;
   extern __shared__ float psm[];   // [2][H][2][64][4]: the normalised weights of one key block
@@ -376,7 +376,8 @@ static int launch_win_mfma(const WinArgs& a, hipStream_t s) {
   auto k = window_attn_mfma_kernel<NDC, NV, HW>;
   if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
     return (int)hipGetLastError();
-  hipLaunchKernelGGL(k, dim3(a.n_items), dim3(256), lds, s, a);
+  const int waves = (a.H + HW - 1) / HW;          // every wave owns HW heads (the last one maybe fewer)
+  hipLaunchKernelGGL(k, dim3(a.n_items), dim3(64 * waves), lds, s, a);
   return (int)hipGetLastError();
 }
 
@@ -432,8 +433,9 @@ K8S_API int k8s_window_attn_mfma(const void* qkv, int qs, const void* kc, const 
   a.BS = BS;
   a.window = window;
   a.scale = scale;
-  const bool wide = H > 8;
-#define K8S_WIN(NDC, NV) (wide ? launch_win_mfma<NDC, NV, 4>(a, s) : launch_win_mfma<NDC, NV, 2>(a, s))
+  // two heads per wave, up to eight waves: two waves per SIMD overlap one's MFMAs with the other's
+  // vector work (measured against four heads per wave at 16 heads: see the design notes)
+#define K8S_WIN(NDC, NV) launch_win_mfma<NDC, NV, 2>(a, s)
   if (D == 64 && V == 64) return K8S_WIN(2, 4);
   if (D == 64 && V == 128) return K8S_WIN(2, 8);
   if (D == 128 && V == 64) return K8S_WIN(4, 4);
