@@ -175,6 +175,10 @@ struct WinArgs {
   uint16_t* out;          // [T][H * V]
   int H, G, BS, window;
   float scale;
+  // split over the keys (steps of few rows): grid.y parts of part_keys keys (a multiple of 32) each
+  int part_keys, n_parts;
+  float* pml;             // [items][parts][H][16][2]: a part's maximum and denominator (log2 units)
+  float* po;              // [items][parts][16][H * V]: a part's share of the output
 };
 
 __device__ __forceinline__ bf16x8 wld16(const uint16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
@@ -200,7 +204,12 @@ __device__ __forceinline__ void win_scores(const bf16x8 (&kf)[2][NDC], const bf1
   }
 }
 
-template <int NDC, int NV, int HW>
+// PHASE 0: both passes over all keys of the tile, bf16 output.  Split over the keys in three launches
+// (part borders count from the tile's first key block: they depend on positions only):
+// PHASE 1: pass 1 over one part, its (maximum, denominator) to pml;
+// PHASE 2: all parts' pml merged, pass 2 over one part, its share of the output to po (fp32);
+// window_attn_merge_kernel then adds the parts' shares.
+template <int NDC, int NV, int HW, int PHASE>
 __global__ void __launch_bounds__(512) window_attn_mfma_kernel(WinArgs a) {
   constexpr int D = NDC * 32, V = NV * 16;
   constexpr float kLog2e = 1.4426950408889634f;
@@ -217,6 +226,10 @@ __global__ void __launch_bounds__(512) window_attn_mfma_kernel(WinArgs a) {
   const int k_lo = max(0, pos0 - a.window + 1), k_hi = pos0 + ntok - 1;
   const float sl2 = a.scale * kLog2e;
   const int* pages = a.bt + (size_t)sg * a.maxb;
+  const int part = PHASE ? blockIdx.y : 0;
+  const int kb_first = (k_lo & ~31) + part * a.part_keys;
+  const int kb_last = PHASE ? min(k_hi, kb_first + a.part_keys - 1) : k_hi;
+  if (kb_first > k_hi) return;                     // an empty part (the whole workgroup leaves)
   bf16x8 qf[HW][NDC];
   float m2[HW], l[HW], c1[HW], c2[HW], inv_l[HW];
 #pragma unroll
@@ -236,7 +249,8 @@ __global__ void __launch_bounds__(512) window_attn_mfma_kernel(WinArgs a) {
     c2[hh] = hh < nh ? a.r2[h0 + hh] : 0.f;
   }
   // ---- pass 1: maximum and denominator
-  for (int kb = k_lo & ~31; kb <= k_hi; kb += 32) {
+  if (PHASE != 2)
+  for (int kb = kb_first; kb <= kb_last; kb += 32) {
     const int page = pages[kb / a.BS], off = kb % a.BS;
     const uint16_t* kp = a.kc + ((size_t)page * a.BS + off) * NK;
     bf16x8 kf[2][NDC];
@@ -272,10 +286,34 @@ __global__ void __launch_bounds__(512) window_attn_mfma_kernel(WinArgs a) {
   }
 #pragma unroll
   for (int hh = 0; hh < HW; ++hh) {
-    float lt = l[hh];
-    lt += __shfl_xor(lt, 16, 64);
-    lt += __shfl_xor(lt, 32, 64);
-    inv_l[hh] = 1.f / (lt + wexp2(-m2[hh]));     // + the sink
+    if (PHASE != 2) {
+      float lt = l[hh];
+      lt += __shfl_xor(lt, 16, 64);
+      lt += __shfl_xor(lt, 32, 64);
+      l[hh] = lt;
+    } else if (hh < nh) {                          // the parts' statistics, merged in part order
+      float M = 0.f, L = 0.f;
+      for (int p2 = 0; p2 < a.n_parts && (k_lo & ~31) + p2 * a.part_keys <= k_hi; ++p2) {
+        const float* ml = a.pml + ((((size_t)item * a.n_parts + p2) * H + h0 + hh) * 16 + r) * 2;
+        const float mp = ml[0], mn = fmaxf(M, mp);
+        L = L * wexp2(M - mn) + ml[1] * wexp2(mp - mn);
+        M = mn;
+      }
+      m2[hh] = M;
+      l[hh] = L;
+    }
+    inv_l[hh] = 1.f / (l[hh] + wexp2(-m2[hh]));   // + the sink
+  }
+  if (PHASE == 1) {
+    if (hq == 0)
+#pragma unroll
+      for (int hh = 0; hh < HW; ++hh)
+        if (hh < nh) {
+          float* ml = a.pml + ((((size_t)item * a.n_parts + part) * H + h0 + hh) * 16 + r) * 2;
+          ml[0] = m2[hh];
+          ml[1] = l[hh];
+        }
+    return;
   }
   // ---- pass 2: weights, mixed over heads, times the values
   f32x4 o[HW][NV];
@@ -284,7 +322,7 @@ __global__ void __launch_bounds__(512) window_attn_mfma_kernel(WinArgs a) {
 #pragma unroll
     for (int dt = 0; dt < NV; ++dt) o[hh][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   int buf = 0;
-  for (int kb = k_lo & ~31; kb <= k_hi; kb += 32) {
+  for (int kb = kb_first; kb <= kb_last; kb += 32) {
     const int page = pages[kb / a.BS], off = kb % a.BS;
     const uint16_t* kp = a.kc + ((size_t)page * a.BS + off) * NK;
     float* P = psm + (size_t)buf * H * 512;
@@ -361,23 +399,54 @@ __global__ void __launch_bounds__(512) window_attn_mfma_kernel(WinArgs a) {
       for (int i = 0; i < 4; ++i) {
         const int q = 4 * hq + i;
         if (q < ntok) {
-          uint16_t* op = a.out + (size_t)(row0 + q) * H * V + (size_t)(h0 + hh) * V + r;
+          if (PHASE == 2) {
+            float* op = a.po + (((size_t)item * a.n_parts + part) * 16 + q) * H * V + (size_t)(h0 + hh) * V + r;
 #pragma unroll
-          for (int dt = 0; dt < NV; ++dt) op[16 * dt] = f2bf(o[hh][dt][i]);
+            for (int dt = 0; dt < NV; ++dt) op[16 * dt] = o[hh][dt][i];
+          } else {
+            uint16_t* op = a.out + (size_t)(row0 + q) * H * V + (size_t)(h0 + hh) * V + r;
+#pragma unroll
+            for (int dt = 0; dt < NV; ++dt) op[16 * dt] = f2bf(o[hh][dt][i]);
+          }
         }
       }
     }
   }
 }
 
-template <int NDC, int NV, int HW>
-static int launch_win_mfma(const WinArgs& a, hipStream_t s) {
-  const size_t lds = (size_t)2 * a.H * 512 * sizeof(float);
-  auto k = window_attn_mfma_kernel<NDC, NV, HW>;
+// out = the sum of the parts' shares (in part order), one workgroup per tile
+__global__ void __launch_bounds__(256) window_attn_merge_kernel(WinArgs a, int HV) {
+  const int item = blockIdx.x;
+  const int row0 = a.items[item * 4 + 1], ntok = a.items[item * 4 + 2], pos0 = a.items[item * 4 + 3];
+  const int k_lo = max(0, pos0 - a.window + 1), k_hi = pos0 + ntok - 1;
+  const int np = min(a.n_parts, (k_hi - (k_lo & ~31)) / a.part_keys + 1);
+  for (int e = threadIdx.x; e < ntok * HV; e += 256) {
+    const int q = e / HV, c = e - q * HV;
+    float acc = 0.f;
+    for (int p2 = 0; p2 < np; ++p2) acc += a.po[(((size_t)item * a.n_parts + p2) * 16 + q) * HV + c];
+    a.out[(size_t)(row0 + q) * HV + c] = f2bf(acc);
+  }
+}
+
+template <int NDC, int NV, int HW, int PHASE>
+static int launch_win_phase(const WinArgs& a, hipStream_t s) {
+  const size_t lds = PHASE == 1 ? 0 : (size_t)2 * a.H * 512 * sizeof(float);
+  auto k = window_attn_mfma_kernel<NDC, NV, HW, PHASE>;
   if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
     return (int)hipGetLastError();
   const int waves = (a.H + HW - 1) / HW;          // every wave owns HW heads (the last one maybe fewer)
-  hipLaunchKernelGGL(k, dim3(a.n_items), dim3(64 * waves), lds, s, a);
+  hipLaunchKernelGGL(k, dim3(a.n_items, PHASE ? a.n_parts : 1), dim3(64 * waves), lds, s, a);
+  return (int)hipGetLastError();
+}
+
+template <int NDC, int NV, int HW>
+static int launch_win_mfma(const WinArgs& a, hipStream_t s) {
+  if (a.n_parts <= 1) return launch_win_phase<NDC, NV, HW, 0>(a, s);
+  int rc = launch_win_phase<NDC, NV, HW, 1>(a, s);
+  if (rc) return rc;
+  rc = launch_win_phase<NDC, NV, HW, 2>(a, s);
+  if (rc) return rc;
+  hipLaunchKernelGGL(window_attn_merge_kernel, dim3(a.n_items), dim3(256), 0, s, a, a.H * NV * 16);
   return (int)hipGetLastError();
 }
 
@@ -411,10 +480,11 @@ K8S_API int k8s_window_attn_mfma_ok(int H, int G, int D, int V) {
 K8S_API int k8s_window_attn_mfma(const void* qkv, int qs, const void* kc, const void* vt, const int* block_tables,
                                  int maxb, const int* items, int n_items, const float* r1, const float* r2,
                                  const float* talk, void* out, int H, int G, int D, int V, int BS, int window,
-                                 float scale, hipStream_t s) {
+                                 float scale, hipStream_t s, int part_keys, int n_parts, float* pml, float* po) {
   if (n_items <= 0) return 0;
   if (!k8s_window_attn_mfma_ok(H, G, D, V) || BS % 32 || window < 1 || qs % 8 || (D * G) % 8)
     return (int)hipErrorInvalidValue;
+  if (n_parts > 1 && (part_keys < 32 || part_keys % 32 || !pml || !po)) return (int)hipErrorInvalidValue;
   WinArgs a;
   a.qkv = (const uint16_t*)qkv;
   a.qs = qs;
@@ -433,6 +503,10 @@ K8S_API int k8s_window_attn_mfma(const void* qkv, int qs, const void* kc, const 
   a.BS = BS;
   a.window = window;
   a.scale = scale;
+  a.part_keys = n_parts > 1 ? part_keys : 32;
+  a.n_parts = n_parts > 1 ? n_parts : 1;
+  a.pml = pml;
+  a.po = po;
   // two heads per wave, up to eight waves: two waves per SIMD overlap one's MFMAs with the other's
   // vector work (measured against four heads per wave at 16 heads: see the design notes)
 #define K8S_WIN(NDC, NV) launch_win_mfma<NDC, NV, 2>(a, s)

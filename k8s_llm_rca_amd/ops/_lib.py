@@ -107,7 +107,7 @@ _SIGS = {
     "k8s_retention": [P, I, P, P, P, P, P, P, P, I, I, I, I, I, F, F, I, P, I, P, P, I, P, P],
     "k8s_window_kv_write": [P, I, I, I, I, P, P, P, I, I, P, P, I],
     "k8s_window_attn_mfma_ok": [I, I, I, I],
-    "k8s_window_attn_mfma": [P, I, P, P, P, I, P, I, P, P, P, P, I, I, I, I, I, I, F, P],
+    "k8s_window_attn_mfma": [P, I, P, P, P, I, P, I, P, P, P, P, I, I, I, I, I, I, F, P, I, I, P, P],
     "k8s_window_attn_rows": [P, I, P, P, P, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
     "k8s_walks": [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P, P, P, P],
 }

@@ -492,6 +492,8 @@ def window_mfma_ok(H: int, G: int, D: int, V: int, dtype, device) -> bool:
 
 
 WINDOW_TILE = 16    # query tokens per work item of the matrix-core window attention kernel
+WINDOW_PART = 128   # keys per part when a step of few rows is split over the keys too
+WINDOW_SPLIT_ITEMS = 32
 
 
 def window_kv_write(qkv: torch.Tensor, k_off: int, kc: torch.Tensor, vc: torch.Tensor, slots: torch.Tensor,
@@ -537,10 +539,22 @@ def window_attention(qkv: torch.Tensor, H: int, G: int, D: int, V: int, kc: torc
         if vt is not None and window_mfma_ok(H, G, D, V, qkv.dtype, qkv.device) and qkv.stride(0) % 8 == 0:
             assert vt.is_contiguous() and vt.shape[1:] == (G * V, BS) and BS % 32 == 0
             items = seg.tile_items(WINDOW_TILE)
+            n_items = items.shape[0]
+            # steps of few rows (decoding): the keys are split over workgroups as well -- parts of
+            # WINDOW_PART keys counted from each tile's first key block, merged in part order
+            n_parts, pml, po = 1, None, None
+            if n_items <= WINDOW_SPLIT_ITEMS:
+                kmax = max(p + b - a for p, a, b in zip(seg.pos0_host, seg.row0_host[:-1], seg.row0_host[1:]))
+                span = min(int(window) + WINDOW_TILE + 30, -(-kmax // 32) * 32)
+                n_parts = -(-span // WINDOW_PART)
+                if n_parts > 1:
+                    pml = scratch(n_items * n_parts * H * 32, torch.float32, qkv.device)
+                    po = scratch(n_items * n_parts * 16 * H * V, torch.float32, qkv.device)
             check(lib().k8s_window_attn_mfma(ptr(qkv), qkv.stride(0), ptr(kc), ptr(vt), ptr(seg.block_tables),
-                                             seg.block_tables.shape[1], ptr(items), items.shape[0], ptr(r1), ptr(r2),
+                                             seg.block_tables.shape[1], ptr(items), n_items, ptr(r1), ptr(r2),
                                              ptr(talk), ptr(out), H, G, D, V, BS, int(window), float(scale),
-                                             stream_ptr(qkv)), "window_attn_mfma")
+                                             stream_ptr(qkv), WINDOW_PART, n_parts, ptr(pml), ptr(po)),
+                  "window_attn_mfma")
             return out
         check(lib().k8s_window_attn_rows(ptr(qkv), qkv.stride(0), ptr(kc), ptr(vc), ptr(seg.block_tables),
                                          seg.block_tables.shape[1], ptr(seg.row_seg), ptr(seg.seg_row0),
