@@ -84,43 +84,47 @@ __global__ void __launch_bounds__(256) short_conv_kernel(const TA* __restrict__ 
   stm(out, (size_t)r * C + c, act ? silu_f(acc) : acc);
 }
 
-// The same for bf16 rows, eight channels per thread (16-byte loads and stores): C % 8 == 0, xs % 8 == 0.
-__global__ void __launch_bounds__(256) short_conv8_kernel(const uint16_t* __restrict__ x, int xs,
-                                                          const float* __restrict__ w, const float* __restrict__ b,
-                                                          const float* __restrict__ tail,
-                                                          const int* __restrict__ row_seg,
-                                                          const int* __restrict__ seg_row0,
-                                                          const int* __restrict__ seg_pos0,
-                                                          const int* __restrict__ seg_slot, uint16_t* __restrict__ out,
-                                                          int C, int taps, int act) {
-  const int r = blockIdx.x, c = (blockIdx.y * 256 + threadIdx.x) * 8;
+// The same over TILES of consecutive rows of one segment ([n][4]: segment, first row, rows, position
+// of the first row), one workgroup per (tile, 256 channels): the segment's metadata is read once per
+// tile instead of once per row, and a thread slides a window of TAPS - 1 earlier inputs in registers,
+// so every input is loaded once.
+template <int TAPS, typename TA>
+__global__ void __launch_bounds__(256) short_conv_tile_kernel(const TA* __restrict__ x, int xs,
+                                                              const float* __restrict__ w, const float* __restrict__ b,
+                                                              const float* __restrict__ tail,
+                                                              const int* __restrict__ items,
+                                                              const int* __restrict__ seg_row0,
+                                                              const int* __restrict__ seg_pos0,
+                                                              const int* __restrict__ seg_slot, TA* __restrict__ out,
+                                                              int C, int act) {
+  const int it = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
   if (c >= C) return;
-  const int sg = row_seg[r], r0 = seg_row0[sg], p0 = seg_pos0[sg];
-  const float* tl = tail + (size_t)seg_slot[sg] * (taps - 1) * C;
-  float acc[8];
+  const int sg = items[it * 4], row0 = items[it * 4 + 1], ntok = items[it * 4 + 2];
+  const int r0 = seg_row0[sg], p0 = seg_pos0[sg];
+  const float* tl = tail + (size_t)seg_slot[sg] * (TAPS - 1) * C;
+  float wt[TAPS], hist[TAPS];   // hist[k]: the input (TAPS - 1 - k) rows before the current one
 #pragma unroll
-  for (int i = 0; i < 8; ++i) acc[i] = b ? b[c + i] : 0.f;
-  for (int j = 0; j < taps; ++j) {
-    const int rr = r - (taps - 1 - j);
-    float v[8];
+  for (int j = 0; j < TAPS; ++j) wt[j] = w[(size_t)c * TAPS + j];
+#pragma unroll
+  for (int k = 0; k < TAPS - 1; ++k) {
+    const int rr = row0 - (TAPS - 1) + k;
     if (rr >= r0) {
-      const u16x8 raw = *reinterpret_cast<const u16x8*>(x + (size_t)rr * xs + c);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) v[i] = bf2f(raw[i]);
+      hist[k] = ldm(x, (size_t)rr * xs + c);
     } else {
       const int back = r0 - rr;
-      const bool have = p0 - back >= 0;
-      const float* tp = tl + (size_t)(taps - 1 - back) * C + c;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) v[i] = have ? tp[i] : 0.f;
+      hist[k] = (p0 - back >= 0) ? tl[(size_t)(TAPS - 1 - back) * C + c] : 0.f;
     }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] = fmaf(w[(size_t)(c + i) * taps + j], v[i], acc[i]);
   }
-  u16x8 o;
+  const float bias = b ? b[c] : 0.f;
+  for (int q = 0; q < ntok; ++q) {
+    hist[TAPS - 1] = ldm(x, (size_t)(row0 + q) * xs + c);
+    float acc = bias;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) o[i] = f2bf(act ? silu_f(acc[i]) : acc[i]);
-  *reinterpret_cast<u16x8*>(out + (size_t)r * C + c) = o;
+    for (int j = 0; j < TAPS; ++j) acc = fmaf(wt[j], hist[j], acc);
+    stm(out, (size_t)(row0 + q) * C + c, act ? silu_f(acc) : acc);
+#pragma unroll
+    for (int j = 0; j < TAPS - 1; ++j) hist[j] = hist[j + 1];
+  }
 }
 
 // After the convolution of a step: the slot's tail becomes the last taps - 1 inputs up to the
@@ -450,22 +454,32 @@ using namespace k8s;
 
 K8S_API int k8s_short_conv(const void* x, int xs, int xdt, const float* w, const float* b, float* tail,
                            const int* row_seg, const int* seg_row0, const int* seg_pos0, const int* seg_slot,
-                           void* out, int T, int n_seg, int C, int taps, int act, int odt, hipStream_t s) {
+                           void* out, int T, int n_seg, int C, int taps, int act, int odt, hipStream_t s,
+                           const int* items, int n_items) {
   if (T <= 0) return 0;
   if (taps < 1 || taps > 16 || xdt != odt) return (int)hipErrorInvalidValue;
   const dim3 g1(T, (C + 255) / 256), g2(n_seg, (C + 255) / 256);
-  const bool vec = odt == 0 && C % 8 == 0 && xs % 8 == 0 && ((uintptr_t)x & 15) == 0;
+  const bool tiles = items != nullptr && n_items > 0 && taps >= 2 && taps <= 4;
+  const dim3 gt(n_items > 0 ? n_items : 1, (C + 255) / 256);
+#define K8S_CONV_T(TP)                                                                                          \
+  hipLaunchKernelGGL((short_conv_tile_kernel<TP, TA>), gt, dim3(256), 0, s, (const TA*)x, xs, w, b, tail, items, \
+                     seg_row0, seg_pos0, seg_slot, (TA*)out, C, act)
   K8S_MDT(odt, {
-    if (vec)
-      hipLaunchKernelGGL(short_conv8_kernel, dim3(T, (C / 8 + 255) / 256), dim3(256), 0, s, (const uint16_t*)x, xs, w,
-                         b, tail, row_seg, seg_row0, seg_pos0, seg_slot, (uint16_t*)out, C, taps, act);
-    else
+    if (tiles && taps == 2) {
+      K8S_CONV_T(2);
+    } else if (tiles && taps == 3) {
+      K8S_CONV_T(3);
+    } else if (tiles) {
+      K8S_CONV_T(4);
+    } else {
       hipLaunchKernelGGL((short_conv_kernel<TA>), g1, dim3(256), 0, s, (const TA*)x, xs, w, b, tail, row_seg, seg_row0,
                          seg_pos0, seg_slot, (TA*)out, C, taps, act);
+    }
     if (taps > 1)
       hipLaunchKernelGGL((short_conv_tail_kernel<TA>), g2, dim3(256), 0, s, (const TA*)x, xs, tail, seg_row0,
                          seg_pos0, seg_slot, C, taps);
   });
+#undef K8S_CONV_T
   return (int)hipGetLastError();
 }
 

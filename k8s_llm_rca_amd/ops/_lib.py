@@ -102,7 +102,7 @@ _SIGS = {
     "k8s_ln_residual": [P, P, P, I, P, P, P, P, P, P, P, P, I, I, I, F, P],
     "k8s_depth_mix_ln": [P, I, I, P, P, I, P, P, P, P, I, I, F, P],
     "k8s_softcap": [P, ctypes.c_long, F, F, P],
-    "k8s_short_conv": [P, I, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
+    "k8s_short_conv": [P, I, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P, P, I],
     "k8s_selective_scan": [P, I, P, P, P, I, I, P, P, P, I, P, P, P, P, P, I, I, I, I, P, P, I, P, P, P],
     "k8s_retention": [P, I, P, P, P, P, P, P, P, I, I, I, I, I, F, F, I, P, I, P, P, I, P, P],
     "k8s_window_kv_write": [P, I, I, I, I, P, P, P, I, I, P, P, I],

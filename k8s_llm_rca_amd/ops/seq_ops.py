@@ -371,9 +371,10 @@ def short_conv(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor], tail
         assert x.stride(1) == 1 and w.dtype == torch.float32 and w.is_contiguous() and tail.is_contiguous()
         assert tail.shape[1:] == (taps - 1, C) and 1 <= taps <= 16 and (b is None or b.dtype == torch.float32)
         d = _dt(x.dtype)
+        items = seg.tile_items(WINDOW_TILE)      # rows in tiles of one segment: metadata once per tile
         check(lib().k8s_short_conv(ptr(x), x.stride(0), d, ptr(w), ptr(b), ptr(tail), ptr(seg.row_seg),
                                    ptr(seg.seg_row0), ptr(seg.seg_pos0), ptr(seg.seg_slot), ptr(out), T, seg.n_seg, C,
-                                   taps, int(act), d, stream_ptr(x)), "short_conv")
+                                   taps, int(act), d, stream_ptr(x), ptr(items), items.shape[0]), "short_conv")
         return out
     nt = taps - 1
     xf = x.float()
