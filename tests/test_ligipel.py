@@ -434,7 +434,7 @@ def run_window(backend, q, k, v, r1, r2, talk, win, scale, cuts, BS=32):
     dev, dt = backend
     T, H, D = q.shape
     G, V = k.shape[1], v.shape[2]
-    order = [5, 2, 7, 0, 3, 6, 1, 4]
+    order = [5, 2, 7, 0, 3, 6, 1, 4, 9, 8]
     kc, row = paged(k.reshape(T, G * D), BS, order, dev, dt)
     vc, _ = paged(v.reshape(T, G * V), BS, order, dev, dt)
     vt = None
@@ -464,6 +464,21 @@ def test_window_attention_paged(backend, H, G, D, V, win):
     want = O.window_attention_core(q, k, v, r1, r2, talk, win, 0.3)
     for cuts in [(T,), (3, 1, 1, 60, 2)]:
         close(run_window(backend, q, k, v, r1, r2, talk, win, 0.3, cuts), want, backend[1])
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("H,G,D,V,win", [(16, 2, 128, 128, 200), (8, 1, 128, 64, 90), (8, 4, 64, 64, 50), (6, 2, 64, 128, 130)])
+def test_window_attention_long_portion(backend, H, G, D, V, win):
+    """A portion of many tiles (the kernels that do not split the keys over workgroups), then token by
+    token (the ones that do)."""
+    T = 540
+    b16 = lambda t: t.to(torch.bfloat16).double()  # noqa: E731
+    q, k, v = b16(rnd(T, H, D, seed=1)), b16(rnd(T, G, D, seed=2)), b16(rnd(T, G, V, seed=3))
+    r1, r2 = rnd(H, seed=4, std=0.3) + 0.5, rnd(H, seed=5).abs()
+    talk = torch.eye(H, dtype=DT) + rnd(H, H, seed=6, std=0.3)
+    want = O.window_attention_core(q, k, v, r1, r2, talk, win, D ** -0.5)
+    got = run_window(backend, q, k, v, r1, r2, talk, win, D ** -0.5, (530, 1, 1), BS=64)
+    close(got, want, backend[1])
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
