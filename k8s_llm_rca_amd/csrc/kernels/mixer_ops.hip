@@ -272,7 +272,8 @@ __global__ void __launch_bounds__(128) scan_carry_kernel(const float* __restrict
 //      scaled by D^(-1/2);
 //   2. retention_scan_kernel, one workgroup per (segment, head, block of <= 32 value columns), tokens
 //      in batches of 16 through LDS:  S <- decay S + k v^T;  o = S^T q  (fp32, written raw).
-//      Thread (dg, v) of NDG x VBS owns S[d][v] for d = dg, dg + NDG, ...  state [slots][H][D][V];
+//      Thread (dg, v) of NDG x VBS owns S[d][v] for the DPT consecutive d from dg DPT (its q and k
+//      entries are neighbours in LDS).  state [slots][H][D][V];
 //   3. head_norm_gate_kernel: out = o / rms(o over the head's V) * silu(g).
 __global__ void __launch_bounds__(256) retention_rope_kernel(float* __restrict__ qkvg, int qs,
                                                              const int* __restrict__ positions, int H, int D, int rot,
@@ -343,7 +344,7 @@ __global__ void __launch_bounds__(256) retention_scan_kernel(const float* __rest
   float S[DPT];
 #pragma unroll
   for (int i = 0; i < DPT; ++i) {
-    const int d = dg + i * NDG;
+    const int d = dg * DPT + i;
     S[i] = (own && d < D && !fresh) ? st[(size_t)d * V + v] : 0.f;
   }
   for (int t0 = r0; t0 < r1; t0 += kRetTb) {
@@ -368,7 +369,7 @@ __global__ void __launch_bounds__(256) retention_scan_kernel(const float* __rest
         float acc = 0.f;
 #pragma unroll
         for (int i = 0; i < DPT; ++i) {
-          const int d = dg + i * NDG;
+          const int d = dg * DPT + i;
           if (d < D) {
             S[i] = fmaf(dec, S[i], kq[d] * vv);
             if (MODE != 1) acc = fmaf(S[i], qq[d], acc);
@@ -392,7 +393,7 @@ __global__ void __launch_bounds__(256) retention_scan_kernel(const float* __rest
   if (MODE != 2) {
 #pragma unroll
     for (int i = 0; i < DPT; ++i) {
-      const int d = dg + i * NDG;
+      const int d = dg * DPT + i;
       if (own && d < D) st[(size_t)d * V + v] = S[i];
     }
   }
