@@ -796,3 +796,32 @@ def test_config_round_trip_registry_and_replay(tmp_path):
     assert rel_err(torch.from_numpy(got[1]), want[[2]]) < 3e-5
     assert rel_err(torch.from_numpy(got[2]), want[[39]]) < 3e-5
     assert eng.kv.free_blocks == 2 and eng.states.free_slots == 4
+
+
+def test_trace_run_command_line(tmp_path):
+    """``bin/trace_run`` as a program: a checkpoint folder, steps on standard input, logits files out."""
+    import os
+    import subprocess
+    import sys
+    import numpy as np
+    from k8s_llm_rca_amd.models.ligipel import save_checkpoint
+    d = config([(ret(2, 4, 6, rot_dims=4), None), (parallel(left(2, 1, 4, 6, 5), right(12, 3, 2, 3)), moe(3, 2, 8, 0))],
+               width=24, vocab=50)
+    W = weights(d, 30)
+    path = str(tmp_path / "ckpt")
+    save_checkpoint(LigipelConfig.from_json(d, "x"), W, path)
+    t = toks(12, d["vocab"], 31)
+    steps = [{"step": 0, "entries": [{"id": "q", "tokens": t[:9], "want": [8]}], "end": []},
+             {"step": 1, "entries": [{"id": "q", "tokens": t[9:10], "want": [0]}], "end": []},
+             {"step": 2, "entries": [{"id": "q", "tokens": t[10:], "want": [0, 1]}], "end": ["q"]}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = str(tmp_path / "out")
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", path, "--dtype", "float32",
+                        "--out", out, "--max-tokens", "64", "--device", "cpu"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [ln for ln in r.stdout.split("\n") if ln.startswith("done")] == ["done 0", "done 1", "done 2"]
+    want = O.forward(d, W, t).float()
+    got = torch.cat([torch.from_numpy(np.fromfile(f"{out}/{i}.f32", dtype="<f4").reshape(-1, d["vocab"]))
+                     for i in range(3)])
+    assert rel_err(got, want[[8, 9, 10, 11]]) < 3e-5
