@@ -21,6 +21,21 @@ __device__ __forceinline__ void stx<float>(float* p, size_t i, float v) { p[i] =
 template <>
 __device__ __forceinline__ void stx<uint16_t>(uint16_t* p, size_t i, float v) { p[i] = f2bf(v); }
 
+// eight consecutive elements (the index a multiple of 8): one 16-byte load for bf16, two for fp32
+__device__ __forceinline__ void ld8(const uint16_t* p, size_t i, float (&v)[8]) {
+  const u16x8 raw = *reinterpret_cast<const u16x8*>(p + i);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) v[k] = bf2f(raw[k]);
+}
+__device__ __forceinline__ void ld8(const float* p, size_t i, float (&v)[8]) {
+  const f32x4 a = *reinterpret_cast<const f32x4*>(p + i), b = *reinterpret_cast<const f32x4*>(p + i + 4);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    v[k] = a[k];
+    v[4 + k] = b[k];
+  }
+}
+
 // PolyNorm: out = a N(z) + b N(z^2) + c N(z^3) + e, N(v) = v / sqrt(mean(v^2) + eps)
 // over the row; z fp32 [T][F], coef = (a, b, c, e).
 template <typename TW, typename TA>
@@ -83,14 +98,14 @@ __global__ void __launch_bounds__(256) router_kernel(const TA* __restrict__ h, c
       for (int j = 0; j < 16; ++j) acc[j] = 0.f;
       for (int c = lane * 8; c < W; c += 512) {
         float hv[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) hv[i] = ldx(h, (size_t)t * W + c + i);
+        ld8(h, (size_t)t * W + c, hv);
 #pragma unroll
         for (int j = 0; j < 16; ++j)
           if (e0 + j < E) {
-            const size_t wo = (size_t)(e0 + j) * W + c;
+            float wv8[8];
+            ld8(wr, (size_t)(e0 + j) * W + c, wv8);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) acc[j] = fmaf(hv[i], ldx(wr, wo + i), acc[j]);
+            for (int i = 0; i < 8; ++i) acc[j] = fmaf(hv[i], wv8[i], acc[j]);
           }
       }
 #pragma unroll

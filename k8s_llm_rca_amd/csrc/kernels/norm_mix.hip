@@ -26,10 +26,10 @@ __device__ __forceinline__ void stn<uint16_t>(uint16_t* p, size_t i, float v) { 
 // mean and 1 / sqrt(var + eps) of the LDS row (all threads get both)
 __device__ __forceinline__ void row_stats(const float* row, int W, float eps, float* red, float& mean, float& rstd) {
   float s = 0.f;
-  for (int c = threadIdx.x; c < W; c += 256) s += row[c];
+  for (int c = threadIdx.x; c < W; c += blockDim.x) s += row[c];
   mean = block_sum(s, red) / (float)W;
   float q = 0.f;
-  for (int c = threadIdx.x; c < W; c += 256) {
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
     const float d = row[c] - mean;
     q = fmaf(d, d, q);
   }
@@ -39,27 +39,27 @@ __device__ __forceinline__ void row_stats(const float* row, int W, float eps, fl
 // 1 / sqrt(mean(v^2) + eps) of a global fp32 row
 __device__ __forceinline__ float row_rrms(const float* v, int W, float eps, float* red) {
   float q = 0.f;
-  for (int c = threadIdx.x; c < W; c += 256) q = fmaf(v[c], v[c], q);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) q = fmaf(v[c], v[c], q);
   return 1.f / sqrtf(block_sum(q, red) / (float)W + eps);
 }
 
 template <typename TA>
-__global__ void __launch_bounds__(256) layernorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+__global__ void __launch_bounds__(1024) layernorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                         const float* __restrict__ b, TA* __restrict__ out, int W,
                                                         float eps) {
   extern __shared__ float row[];
   __shared__ float red[16];
   const size_t o = (size_t)blockIdx.x * W;
-  for (int c = threadIdx.x; c < W; c += 256) row[c] = x[o + c];
+  for (int c = threadIdx.x; c < W; c += blockDim.x) row[c] = x[o + c];
   __syncthreads();
   float mean, rstd;
   row_stats(row, W, eps, red, mean, rstd);
-  for (int c = threadIdx.x; c < W; c += 256) stn(out, o + c, (row[c] - mean) * rstd * w[c] + b[c]);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) stn(out, o + c, (row[c] - mean) * rstd * w[c] + b[c]);
 }
 
 // x_out = LN(embed[id]; w, b); optionally h = LN(x_out; nw, nb).
 template <typename TE, typename TA>
-__global__ void __launch_bounds__(256) embed_ln_kernel(const int* __restrict__ ids, const TE* __restrict__ embed,
+__global__ void __launch_bounds__(1024) embed_ln_kernel(const int* __restrict__ ids, const TE* __restrict__ embed,
                                                        const float* __restrict__ w, const float* __restrict__ b,
                                                        float* __restrict__ x_out, const float* __restrict__ nw,
                                                        const float* __restrict__ nb, TA* __restrict__ h, int W,
@@ -67,12 +67,12 @@ __global__ void __launch_bounds__(256) embed_ln_kernel(const int* __restrict__ i
   extern __shared__ float row[];
   __shared__ float red[16];
   const size_t o = (size_t)blockIdx.x * W, e0 = (size_t)ids[blockIdx.x] * W;
-  for (int c = threadIdx.x; c < W; c += 256) row[c] = ldn(embed, e0 + c);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) row[c] = ldn(embed, e0 + c);
   __syncthreads();
   float mean, rstd;
   row_stats(row, W, eps, red, mean, rstd);
   __syncthreads();
-  for (int c = threadIdx.x; c < W; c += 256) {
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
     const float v = (row[c] - mean) * rstd * w[c] + b[c];
     row[c] = v;
     x_out[o + c] = v;
@@ -80,13 +80,13 @@ __global__ void __launch_bounds__(256) embed_ln_kernel(const int* __restrict__ i
   if (nw == nullptr) return;
   __syncthreads();
   row_stats(row, W, eps, red, mean, rstd);
-  for (int c = threadIdx.x; c < W; c += 256) stn(h, o + c, (row[c] - mean) * rstd * nw[c] + nb[c]);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) stn(h, o + c, (row[c] - mean) * rstd * nw[c] + nb[c]);
 }
 
 // dst = src + LN(u; w, b); u = y (mode 0), (unit_rms(y) wl + unit_rms(y2) wr) / 2 (mode 1), y + y2 (mode 2).
 // Optionally h = LN(dst; nw, nb).
 template <typename TA>
-__global__ void __launch_bounds__(256) ln_residual_kernel(const float* src, const float* __restrict__ y,
+__global__ void __launch_bounds__(1024) ln_residual_kernel(const float* src, const float* __restrict__ y,
                                                           const float* __restrict__ y2, int mode,
                                                           const float* __restrict__ wl, const float* __restrict__ wr,
                                                           const float* __restrict__ w, const float* __restrict__ b,
@@ -98,17 +98,17 @@ __global__ void __launch_bounds__(256) ln_residual_kernel(const float* src, cons
   const size_t o = (size_t)blockIdx.x * W;
   if (mode == 1) {
     const float ra = row_rrms(y + o, W, eps, red), rb = row_rrms(y2 + o, W, eps, red);
-    for (int c = threadIdx.x; c < W; c += 256) row[c] = 0.5f * (y[o + c] * ra * wl[c] + y2[o + c] * rb * wr[c]);
+    for (int c = threadIdx.x; c < W; c += blockDim.x) row[c] = 0.5f * (y[o + c] * ra * wl[c] + y2[o + c] * rb * wr[c]);
   } else if (mode == 2) {
-    for (int c = threadIdx.x; c < W; c += 256) row[c] = y[o + c] + y2[o + c];
+    for (int c = threadIdx.x; c < W; c += blockDim.x) row[c] = y[o + c] + y2[o + c];
   } else {
-    for (int c = threadIdx.x; c < W; c += 256) row[c] = y[o + c];
+    for (int c = threadIdx.x; c < W; c += blockDim.x) row[c] = y[o + c];
   }
   __syncthreads();
   float mean, rstd;
   row_stats(row, W, eps, red, mean, rstd);
   __syncthreads();
-  for (int c = threadIdx.x; c < W; c += 256) {
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
     const float v = src[o + c] + ((row[c] - mean) * rstd * w[c] + b[c]);
     row[c] = v;
     dst[o + c] = v;
@@ -116,12 +116,12 @@ __global__ void __launch_bounds__(256) ln_residual_kernel(const float* src, cons
   if (nw == nullptr) return;
   __syncthreads();
   row_stats(row, W, eps, red, mean, rstd);
-  for (int c = threadIdx.x; c < W; c += 256) stn(h, o + c, (row[c] - mean) * rstd * nw[c] + nb[c]);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) stn(h, o + c, (row[c] - mean) * rstd * nw[c] + nb[c]);
 }
 
 // a = sum_{j < n} coef[j] * stack[j][row]; h = LN(a; w, b).  stack: [n][T][W]; rows: optional gather.
 template <typename TA>
-__global__ void __launch_bounds__(256) depth_mix_ln_kernel(const float* __restrict__ stack, size_t plane, int n,
+__global__ void __launch_bounds__(1024) depth_mix_ln_kernel(const float* __restrict__ stack, size_t plane, int n,
                                                            const float* __restrict__ coef,
                                                            const int* __restrict__ rows, float* __restrict__ a_out,
                                                            const float* __restrict__ w, const float* __restrict__ b,
@@ -130,7 +130,7 @@ __global__ void __launch_bounds__(256) depth_mix_ln_kernel(const float* __restri
   __shared__ float red[16];
   const size_t r = rows ? (size_t)rows[blockIdx.x] : (size_t)blockIdx.x;
   const size_t o = (size_t)blockIdx.x * W;
-  for (int c = threadIdx.x; c < W; c += 256) {
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float a = 0.f;
     for (int j = 0; j < n; ++j) a = fmaf(coef[j], stack[(size_t)j * plane + r * W + c], a);
     row[c] = a;
@@ -139,7 +139,7 @@ __global__ void __launch_bounds__(256) depth_mix_ln_kernel(const float* __restri
   __syncthreads();
   float mean, rstd;
   row_stats(row, W, eps, red, mean, rstd);
-  for (int c = threadIdx.x; c < W; c += 256) stn(h, o + c, (row[c] - mean) * rstd * w[c] + b[c]);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) stn(h, o + c, (row[c] - mean) * rstd * w[c] + b[c]);
 }
 
 __global__ void __launch_bounds__(256) softcap_kernel(float* __restrict__ z, size_t n, float scale, float cap) {
@@ -163,12 +163,14 @@ using namespace k8s;
   }
 
 static inline bool row_fits(int W) { return W > 0 && (size_t)W * sizeof(float) <= 64 * 1024; }
+// threads per row: few rows (decoding) leave most of the chip idle, so each row gets a wider workgroup
+static inline int row_threads(int rows, int W) { return rows <= 256 && W >= 1024 ? 1024 : 256; }
 
 K8S_API int k8s_layernorm(const float* x, const float* w, const float* b, void* out, int T, int W, float eps, int dt,
                           hipStream_t s) {
   if (T <= 0) return 0;
   if (!row_fits(W)) return (int)hipErrorInvalidValue;
-  K8S_ODT(dt, hipLaunchKernelGGL((layernorm_kernel<TA>), dim3(T), dim3(256), W * sizeof(float), s, x, w, b, (TA*)out,
+  K8S_ODT(dt, hipLaunchKernelGGL((layernorm_kernel<TA>), dim3(T), dim3(row_threads(T, W)), W * sizeof(float), s, x, w, b, (TA*)out,
                                  W, eps));
   return (int)hipGetLastError();
 }
@@ -178,10 +180,10 @@ K8S_API int k8s_embed_ln(const int* ids, const void* embed, int edt, const float
   if (T <= 0) return 0;
   if (!row_fits(W)) return (int)hipErrorInvalidValue;
   if (edt == 0) {
-    K8S_ODT(dt, hipLaunchKernelGGL((embed_ln_kernel<uint16_t, TA>), dim3(T), dim3(256), W * sizeof(float), s, ids,
+    K8S_ODT(dt, hipLaunchKernelGGL((embed_ln_kernel<uint16_t, TA>), dim3(T), dim3(row_threads(T, W)), W * sizeof(float), s, ids,
                                    (const uint16_t*)embed, w, b, x_out, nw, nb, (TA*)h, W, eps));
   } else {
-    K8S_ODT(dt, hipLaunchKernelGGL((embed_ln_kernel<float, TA>), dim3(T), dim3(256), W * sizeof(float), s, ids,
+    K8S_ODT(dt, hipLaunchKernelGGL((embed_ln_kernel<float, TA>), dim3(T), dim3(row_threads(T, W)), W * sizeof(float), s, ids,
                                    (const float*)embed, w, b, x_out, nw, nb, (TA*)h, W, eps));
   }
   return (int)hipGetLastError();
@@ -192,7 +194,7 @@ K8S_API int k8s_ln_residual(const float* src, const float* y, const float* y2, i
                             const float* nb, void* h, int dt, int T, int W, float eps, hipStream_t s) {
   if (T <= 0) return 0;
   if (!row_fits(W) || (mode != 0 && y2 == nullptr) || (mode == 1 && (!wl || !wr))) return (int)hipErrorInvalidValue;
-  K8S_ODT(dt, hipLaunchKernelGGL((ln_residual_kernel<TA>), dim3(T), dim3(256), W * sizeof(float), s, src, y, y2, mode,
+  K8S_ODT(dt, hipLaunchKernelGGL((ln_residual_kernel<TA>), dim3(T), dim3(row_threads(T, W)), W * sizeof(float), s, src, y, y2, mode,
                                  wl, wr, w, b, dst, nw, nb, (TA*)h, W, eps));
   return (int)hipGetLastError();
 }
@@ -202,7 +204,7 @@ K8S_API int k8s_depth_mix_ln(const float* stack, int T, int n, const float* coef
                              hipStream_t s) {
   if (R <= 0) return 0;
   if (!row_fits(W) || n < 1) return (int)hipErrorInvalidValue;
-  K8S_ODT(dt, hipLaunchKernelGGL((depth_mix_ln_kernel<TA>), dim3(R), dim3(256), W * sizeof(float), s, stack,
+  K8S_ODT(dt, hipLaunchKernelGGL((depth_mix_ln_kernel<TA>), dim3(R), dim3(row_threads(R, W)), W * sizeof(float), s, stack,
                                  (size_t)T * W, n, coef, rows, a_out, w, b, (TA*)h, W, eps));
   return (int)hipGetLastError();
 }

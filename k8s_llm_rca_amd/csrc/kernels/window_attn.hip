@@ -420,7 +420,7 @@ __global__ void __launch_bounds__(256) window_attn_merge_kernel(WinArgs a, int H
   const int row0 = a.items[item * 4 + 1], ntok = a.items[item * 4 + 2], pos0 = a.items[item * 4 + 3];
   const int k_lo = max(0, pos0 - a.window + 1), k_hi = pos0 + ntok - 1;
   const int np = min(a.n_parts, (k_hi - (k_lo & ~31)) / a.part_keys + 1);
-  for (int e = threadIdx.x; e < ntok * HV; e += 256) {
+  for (int e = blockIdx.y * 256 + threadIdx.x; e < ntok * HV; e += gridDim.y * 256) {
     const int q = e / HV, c = e - q * HV;
     float acc = 0.f;
     for (int p2 = 0; p2 < np; ++p2) acc += a.po[(((size_t)item * a.n_parts + p2) * 16 + q) * HV + c];
@@ -446,7 +446,7 @@ static int launch_win_mfma(const WinArgs& a, hipStream_t s) {
   if (rc) return rc;
   rc = launch_win_phase<NDC, NV, HW, 2>(a, s);
   if (rc) return rc;
-  hipLaunchKernelGGL(window_attn_merge_kernel, dim3(a.n_items), dim3(256), 0, s, a, a.H * NV * 16);
+  hipLaunchKernelGGL(window_attn_merge_kernel, dim3(a.n_items, 16), dim3(256), 0, s, a, a.H * NV * 16);
   return (int)hipGetLastError();
 }
 
