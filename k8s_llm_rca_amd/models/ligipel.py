@@ -38,6 +38,7 @@ from ..ops import norm as N
 from ..ops import seq_ops as S
 from ..ops.linear import linear, linear_f32out, swiglu_gemm
 from ..parallel.groups import ParallelContext, single
+from .moe import MoELayerSet
 
 RENORM_EPS = 1e-20      # router: chosen scores are divided by their sum + RENORM_EPS
 
@@ -384,9 +385,17 @@ class LigipelModel:
                 and M.grouped_big_ok(rows, W, f.ff, False)):
             # prefill sizes: the grouped MFMA GEMM with the gated unit in its epilogue (gate_up never written)
             act = M.grouped_big(xp, L["w13"], offsets, silu=True)
+        elif xp.is_cuda and xp.dtype == torch.bfloat16 and rows <= MoELayerSet.GLDS_MAX_ROWS:
+            # decode sizes: the weight-streaming kernels the Mixtral block runs there (LDS-DMA strips for
+            # gate_up; the down projection below with its K split over workgroups)
+            gu = M.grouped_gemm(xp, L["w13"], offsets, glds=MoELayerSet.GLDS_UP[0], splits=MoELayerSet.GLDS_UP[1])
+            act = M.glu_clamp(gu, 1.0, math.inf, 0.0)
         else:
             act = M.glu_clamp(M.grouped_auto(xp, L["w13"], offsets), 1.0, math.inf, 0.0)  # silu(gate) * up
-        yp = M.grouped_auto(act, L["w2"], offsets)
+        if xp.is_cuda and xp.dtype == torch.bfloat16 and rows <= MoELayerSet.SPLIT_MAX_ROWS:
+            yp = M.grouped_gemm(act, L["w2"], offsets, splits=MoELayerSet.DOWN_SPLITS)
+        else:
+            yp = M.grouped_auto(act, L["w2"], offsets)
         routed = M.combine_f32(yp, inv, T, f.top, w)
         shared = None
         if f.shared_ff:
