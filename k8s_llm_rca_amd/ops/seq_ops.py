@@ -125,6 +125,7 @@ class SegMeta:
 
 SCAN_CHUNK = 64     # rows per chunk of the time-parallel minGRU
 SSM_CHUNK = 64      # rows per chunk of the time-parallel selective scan and retention
+SEQ_FILL_LANES = 1 << 18   # sequential lanes (segments x channels) from which the chunk-parallel form stops paying
 
 
 def _dt(t: torch.dtype) -> int:
@@ -408,7 +409,8 @@ def selective_scan(xc: torch.Tensor, dtp: torch.Tensor, dt_bias: torch.Tensor, d
         assert A.dtype == D.dtype == dt_bias.dtype == torch.float32 and A.is_contiguous()
         # long portions: chunks run in parallel (a pass from zero states, a carry over the chunks, the
         # chunks again from their start states); short ones token by token
-        cr = seg.chunk_ranges(SSM_CHUNK, 2 * SSM_CHUNK)
+        # (with many sequences the token-by-token kernel already fills the chip, at half the exponentials)
+        cr = seg.chunk_ranges(SSM_CHUNK, 2 * SSM_CHUNK) if seg.n_seg * C < SEQ_FILL_LANES else None
         chunks, c0, cs, csd, nch = None, None, None, None, 0
         if cr is not None:
             chunks, c0 = cr
@@ -448,7 +450,7 @@ def retention(qkvg: torch.Tensor, H: int, D: int, V: int, decay: torch.Tensor, r
         oraw = scratch(T * H * V, torch.float32, qkvg.device)
         # long portions: chunks in parallel (end states from zero, a carry over the chunks, the chunks
         # again from their start states); short ones token by token
-        cr = seg.chunk_ranges(SSM_CHUNK, 2 * SSM_CHUNK)
+        cr = seg.chunk_ranges(SSM_CHUNK, 2 * SSM_CHUNK) if seg.n_seg * H * V * 8 < SEQ_FILL_LANES else None
         chunks, c0, cs, nch = None, None, None, 0
         if cr is not None:
             chunks, c0 = cr
